@@ -12,7 +12,9 @@
 // (attention.rs:225-233) and, when a window w is given, > p - w; a position encoding that works
 // on the scores gives `slopes` (one float per query head; the reference has none): the score of
 // key position u for a query at position p then gets slope * (u - p) added, in float32, before
-// the softmax; softmax statistics (running
+// the softmax; `head_scales` (one float per query head, or null) multiply the score scale of
+// their head, and with softcap c > 0 the scaled score becomes c * tanh(score / c) before bias
+// and softmax, all in float32; softmax statistics (running
 // maximum m, denominator l, unnormalised accumulator) are float32; partitions of a long
 // context are merged with weights e^(m_i - max m) over the non-empty ones (metal:276-304).
 //
@@ -31,7 +33,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const TX* __restrict__ k_pages, const TX* __restrict__ v_pages,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, int nh, int nkv, int d, int page_size, float scale,
-    int window, const float* __restrict__ slopes) {
+    int window, const float* __restrict__ slopes, const float* __restrict__ head_scales,
+    float softcap) {
   extern __shared__ float smem[];
   float* q_s = smem;                          // d
   float* p_s = smem + d;                      // 64
@@ -42,6 +45,8 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
   const int kvh = h / (nh / nkv);
   const float slope = slopes ? slopes[h] : 0.f;
   const int* table = block_tables + (long long)seq * max_pages;
+  if (head_scales) scale *= head_scales[h];
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   for (int j = lane; j < d; j += 64) q_s[j] = ld(q + (long long)t * q_stride + h * d + j) * scale;
   __syncthreads();
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -60,6 +65,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
       const TX* kp = k_pages + ((page * nkv + kvh) * page_size + off) * d;
       float dot = 0.f;
       for (int j = 0; j < d; ++j) dot = fmaf(q_s[j], ld(kp + j), dot);
+      if (softcap > 0.f) dot = softcap * tanhf(dot * inv_cap);
       s = dot + slope * (float)(kpos - pos);
       vbase = (page * nkv + kvh) * (long long)d * page_size + off;
     }
@@ -97,7 +103,7 @@ RLIS_API int rlis_attn_generic(const void* q, int dtype, long long q_stride, voi
                                const int* block_tables, int max_pages, const int* seq_of_token,
                                const int* positions, int T, int nh, int nkv, int d, int page_size,
                                float scale, int window, const float* slopes,
-                               hipStream_t stream) {
+                               const float* head_scales, float softcap, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_generic: bad sizes");
   RLIS_REQUIRE(nh % nkv == 0, "attn_generic: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
@@ -111,7 +117,7 @@ RLIS_API int rlis_attn_generic(const void* q, int dtype, long long q_stride, voi
   attn_generic_kernel<TX, DPL><<<grid, 64, smem, stream>>>(                                    \
       (const TX*)q, q_stride, (TX*)out, out_stride, (const TX*)k_pages, (const TX*)v_pages,    \
       block_tables, max_pages, seq_of_token, positions, nh, nkv, d, page_size, scale, window,  \
-      slopes)
+      slopes, head_scales, softcap)
 #define BY_DPL(TX)                         \
   do {                                     \
     if (dpl <= 1) LAUNCH(TX, 1);           \
@@ -166,7 +172,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const TX* __restrict__ v_pages, const int* __restrict__ block_tables, int max_pages,
     const int* __restrict__ ctx_lens, const int* __restrict__ token_rows, int nh, int nkv, int d,
     int page_size, float scale, int window, int splits, int chunks_per_kv, int part_keys,
-    int max_parts, const float* __restrict__ slopes) {
+    int max_parts, const float* __restrict__ slopes, const float* __restrict__ head_scales,
+    float softcap) {
   extern __shared__ float smem[];
   float* q_s = smem;                     // G * d
   float* p_s = q_s + G * d;              // 4 waves * G * 64
@@ -190,7 +197,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
 
   for (int i = tid; i < G * d; i += 256) {
     const int hh = min(i / d, gn - 1), j = i % d;
-    q_s[i] = ld(q + (long long)row * q_stride + (h0 + hh) * d + j) * scale;
+    q_s[i] = ld(q + (long long)row * q_stride + (h0 + hh) * d + j) * scale *
+             (head_scales ? head_scales[h0 + hh] : 1.0f);
   }
   __syncthreads();
 
@@ -242,7 +250,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     float corr[G];
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
-      const float sv = valid ? s[hh] + slope[hh] * (float)(kpos - (ctx - 1)) : -INFINITY;
+      const float capped = softcap > 0.f ? softcap * tanhf(s[hh] / softcap) : s[hh];
+      const float sv = valid ? capped + slope[hh] * (float)(kpos - (ctx - 1)) : -INFINITY;
       const float m_new = fmaxf(m[hh], wave_max(sv));
       const float p = valid ? expf(sv - m_new) : 0.f;
       corr[hh] = (m[hh] == -INFINITY) ? 0.f : expf(m[hh] - m_new);
@@ -503,7 +512,8 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
                          const void* v_pages, const int* block_tables, int max_pages,
                          const int* ctx_lens, const int* token_rows, int S, int nh, int nkv, int d,
                          int page_size, float scale, int window, int splits, int part_keys,
-                         int max_parts, const float* slopes, hipStream_t stream) {
+                         int max_parts, const float* slopes, const float* head_scales,
+                         float softcap, hipStream_t stream) {
   const int g = nh / nkv;
   const int chunks = ceil_div(g, G);
   dim3 grid(nkv * chunks, S, splits);
@@ -515,7 +525,7 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
   attn_decode_kernel<TX, G, DPL><<<grid, 256, smem, stream>>>(                                 \
       (const TX*)q, q_stride, (TX*)out, out_stride, part_ml, part_acc, (const TX*)k_pages,     \
       (const TX*)v_pages, block_tables, max_pages, ctx_lens, token_rows, nh, nkv, d, page_size, \
-      scale, window, splits, chunks, part_keys, max_parts, slopes)
+      scale, window, splits, chunks, part_keys, max_parts, slopes, head_scales, softcap)
   if (dpl <= 1) LAUNCH(1);
   else if (dpl <= 2) LAUNCH(2);
   else LAUNCH(4);
@@ -534,7 +544,7 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
                               int max_pages, const int* ctx_lens, const int* token_rows, int S,
                               int nh, int nkv, int d, int page_size, float scale, int window,
                               int splits, int part_keys, int max_parts, const float* slopes,
-                              hipStream_t stream) {
+                              const float* head_scales, float softcap, hipStream_t stream) {
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode: bad sizes");
   RLIS_REQUIRE(part_keys >= 64 && part_keys % 64 == 0 && max_parts >= 1 && splits <= max_parts,
                "attn_decode: partitions of %d keys (a multiple of 64), %d deep of at most %d",
@@ -554,22 +564,22 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
       rc = launch_decode<TX, 1>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, stream);               \
+                                slopes, head_scales, softcap, stream);               \
     else if (g == 2)                                                                             \
       rc = launch_decode<TX, 2>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, stream);               \
+                                slopes, head_scales, softcap, stream);               \
     else if (g <= 4)                                                                             \
       rc = launch_decode<TX, 4>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, stream);               \
+                                slopes, head_scales, softcap, stream);               \
     else                                                                                         \
       rc = launch_decode<TX, 8>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, stream);               \
+                                slopes, head_scales, softcap, stream);               \
   } while (0)
   if (dtype == RLIS_F32) BY_G(float);
   else if (dtype == RLIS_BF16) BY_G(bf16_t);

@@ -21,25 +21,38 @@ void rlis_set_error(const char* fmt, ...) {
 RLIS_API const char* rlis_last_error() { return g_err; }
 
 // ------------------------------------------------------------------------ embedding
+// out[t] = table[ids[t]] * scale (+ learned[positions[t]] when a table of learned position
+// vectors is given: added as it is, in float32).
 template <typename TW>
 __global__ void embed_kernel(float* __restrict__ out, const TW* __restrict__ table,
-                             const int* __restrict__ ids, int H, float scale) {
+                             const int* __restrict__ ids, int H, float scale,
+                             const TW* __restrict__ learned, const int* __restrict__ positions) {
   const int t = blockIdx.x;
   const long long row = ids[t];
   const TW* src = table + row * H;
   float* dst = out + (long long)t * H;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ld(src + j) * scale;
+  if (learned) {
+    const TW* add = learned + (long long)positions[t] * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ld(src + j) * scale + ld(add + j);
+  } else {
+    for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ld(src + j) * scale;
+  }
 }
 
-// out (T,H) f32 <- table[ids] * scale ; ids are checked against V on the host before the call.
+// out (T,H) f32 <- table[ids] * scale (+ learned[positions]); ids and positions are checked
+// against the tables' rows on the host before the call.
 RLIS_API int rlis_embed(float* out, const void* table, int table_dtype, const int* ids, int T,
-                        int H, float scale, hipStream_t stream) {
+                        int H, float scale, const void* learned, const int* positions,
+                        hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && H > 0, "embed: bad sizes T=%d H=%d", T, H);
+  RLIS_REQUIRE(!learned || positions, "embed: learned position vectors need positions");
   if (T == 0) return 0;
   if (table_dtype == RLIS_F32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H, scale);
+    embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H, scale,
+                                               (const float*)learned, positions);
   else if (table_dtype == RLIS_BF16)
-    embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H, scale);
+    embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H, scale,
+                                                (const bf16_t*)learned, positions);
   else
     RLIS_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
   RLIS_LAUNCH_CHECK("embed");
@@ -609,6 +622,111 @@ RLIS_API int rlis_weighted_sum(float* out, const void* x, int x_dtype, float a, 
   }
 #undef CASE
   RLIS_LAUNCH_CHECK("weighted_sum");
+  return 0;
+}
+
+// ------------------------------------------------------------- tanh form of GELU
+// y = 0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))), float32 arithmetic, one rounding.
+__device__ __forceinline__ float gelu_tanh_f(float x) {
+  const float inner = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+template <typename TX>
+__global__ void gelu_tanh_kernel(TX* __restrict__ out, const TX* __restrict__ x, long long n) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) st(out + i, gelu_tanh_f(ld(x + i)));
+}
+
+// bfloat16, eight values a thread (16-byte accesses); tanh(z) = 1 - 2 / (exp(2 z) + 1) with the
+// hardware's exponential and reciprocal.
+__global__ void gelu_tanh_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ x,
+                                        long long n8) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n8; i += stride) {
+    const uint4 v = *(const uint4*)(x + i * 8);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float r[2];
+      const float a[2] = {__uint_as_float(w[j] << 16), __uint_as_float(w[j] & 0xffff0000u)};
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float z = 0.7978845608028654f * (a[e] + 0.044715f * a[e] * a[e] * a[e]);
+        // 0.5 (1 + tanh z) = 1 / (1 + exp(-2 z))
+        const float ex = __builtin_amdgcn_exp2f(-2.0f * 1.4426950408889634f * z);
+        r[e] = a[e] * __builtin_amdgcn_rcpf(1.0f + ex);
+      }
+      o[j] = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
+    }
+    *(uint4*)(out + i * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+RLIS_API int rlis_gelu_tanh(void* out, const void* x, int dtype, long long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (dtype == RLIS_BF16 && n % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)x % 16) == 0) {
+    const long long n8 = n / 8;
+    const int blocks8 = (int)(ceil_div_ll(n8, 256) < 16384 ? ceil_div_ll(n8, 256) : 16384);
+    gelu_tanh_bf16x8_kernel<<<blocks8, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, n8);
+    RLIS_LAUNCH_CHECK("gelu_tanh");
+    return 0;
+  }
+  const int blocks = (int)(ceil_div_ll(n, 256) < 8192 ? ceil_div_ll(n, 256) : 8192);
+  if (dtype == RLIS_F32)
+    gelu_tanh_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, n);
+  else if (dtype == RLIS_BF16)
+    gelu_tanh_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, n);
+  else
+    RLIS_REQUIRE(false, "gelu_tanh: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("gelu_tanh");
+  return 0;
+}
+
+// ------------------------------------------------- a learned mix of the layers' results
+// The stream that the next layer reads is a weighted sum of the embedding output and of every
+// layer's result so far.  `hist` holds them, one (T, W) float32 slab per source, `n` elements
+// apart.  This layer's result y = x + delta becomes source `count - 1`; x then becomes
+// sum_j weights[j] * source j over the `count` sources, added in order, all in float32.  With
+// save_input, x itself is stored as source 0 first (the first layer: its input is the embedding
+// output as it is).
+template <typename TW>
+__global__ void depth_mix_kernel(float* __restrict__ x, const float* __restrict__ delta,
+                                 float* __restrict__ hist, long long n, int count,
+                                 const TW* __restrict__ weights, int save_input) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const float in = x[i];
+    const float y = in + delta[i];
+    if (save_input) hist[i] = in;
+    hist[(long long)(count - 1) * n + i] = y;
+    float acc = ld(weights) * (save_input ? in : hist[i]);
+    for (int j = 1; j < count - 1; ++j) acc += ld(weights + j) * hist[(long long)j * n + i];
+    acc += ld(weights + count - 1) * y;
+    x[i] = acc;
+  }
+}
+
+RLIS_API int rlis_depth_mix(float* x, const float* delta, float* hist, long long n, int count,
+                            const void* weights, int weights_dtype, int save_input,
+                            hipStream_t stream) {
+  RLIS_REQUIRE(count >= 2, "depth_mix: %d sources, at least the input and one result", count);
+  RLIS_REQUIRE(!save_input || count == 2, "depth_mix: only the first layer stores its input");
+  if (n <= 0) return 0;
+  const int blocks = (int)(ceil_div_ll(n, 256) < 8192 ? ceil_div_ll(n, 256) : 8192);
+  if (weights_dtype == RLIS_F32)
+    depth_mix_kernel<float><<<blocks, 256, 0, stream>>>(x, delta, hist, n, count,
+                                                        (const float*)weights, save_input);
+  else if (weights_dtype == RLIS_BF16)
+    depth_mix_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, delta, hist, n, count,
+                                                         (const bf16_t*)weights, save_input);
+  else
+    RLIS_REQUIRE(false, "depth_mix: unknown dtype %d", weights_dtype);
+  RLIS_LAUNCH_CHECK("depth_mix");
   return 0;
 }
 

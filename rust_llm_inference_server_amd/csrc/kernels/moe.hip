@@ -5,6 +5,8 @@
 //    largest choice scores, only experts of the `keep` best groups can be chosen (the others
 //    count as minus infinity); the `top` largest choice scores win (the lower index on a tie);
 //    an expert's weight is its s times `scale`, not renormalised.  One wave per token.
+//    Switches: s = softmax(z) over all experts; a group's score the largest choice score in it;
+//    the chosen experts' weights divided by their sum.  A unit's bounded form: see gated_unit.
 //  * moe_sort: the step's (token, choice) pairs ordered by expert, every expert's run padded to
 //    whole tiles of rows, so that a tile has one expert.  Decided on the device: nothing waits
 //    for the host.  Which row of its expert's run a pair gets does not move its result: rows of a
@@ -95,7 +97,21 @@ RLIS_API int rlis_moe_router_logits(const float* resid, const void* ln_w, const 
   return 0;
 }
 
+// What a unit makes of its gate and up products: silu(g) * u, or with limit > 0 the bounded
+// form g' * sigmoid(alpha * g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
+__device__ __forceinline__ float gated_unit(float g, float u, float limit, float alpha) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
+
 // ------------------------------------------------------------------------ route
+// Scores: sigmoid of the logits, or (softmax_scores) their softmax over all experts.  A group's
+// score: the sum of its two largest choice scores, or (group_max) the largest.  Weights: the
+// chosen experts' scores times `scale`, or (renormalise) divided by their sum + 1e-20 first.
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -107,15 +123,27 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
 
 __global__ __launch_bounds__(64) void moe_route_kernel(
     const float* __restrict__ z, long long ldz, const float* __restrict__ correction, int E,
-    int G, int keep, int top, float scale, int* __restrict__ chosen, float* __restrict__ weights) {
+    int G, int keep, int top, float scale, int* __restrict__ chosen, float* __restrict__ weights,
+    int softmax_scores, int group_max, int renormalise) {
   extern __shared__ float sm[];
   float* choice = sm;            // E
   float* gscore = sm + E;        // G
+  float* score = sm + E + G;     // E
   const int t = blockIdx.x, lane = threadIdx.x;
   const int per = E / G;
+  float zmax = -INFINITY, zsum = 1.f;
+  if (softmax_scores) {
+    for (int e = lane; e < E; e += 64) zmax = fmaxf(zmax, z[(long long)t * ldz + e]);
+    zmax = wave_max(zmax);
+    float part = 0.f;
+    for (int e = lane; e < E; e += 64) part += expf(z[(long long)t * ldz + e] - zmax);
+    zsum = wave_sum(part);
+  }
   for (int e = lane; e < E; e += 64) {
-    const float s = 1.0f / (1.0f + expf(-z[(long long)t * ldz + e]));
-    choice[e] = s + correction[e];
+    const float zv = z[(long long)t * ldz + e];
+    const float s = softmax_scores ? expf(zv - zmax) / zsum : 1.0f / (1.0f + expf(-zv));
+    score[e] = s;
+    choice[e] = s + (correction ? correction[e] : 0.f);
   }
   __syncthreads();
   for (int g = lane; g < G; g += 64) {
@@ -124,7 +152,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
       const float c = choice[g * per + i];
       if (c > a) { b = a; a = c; } else if (c > b) { b = c; }
     }
-    gscore[g] = per > 1 ? a + b : a;
+    gscore[g] = (per > 1 && !group_max) ? a + b : a;
   }
   __syncthreads();
   // the groups that stay: `keep` rounds of the largest score, lower index on a tie
@@ -153,25 +181,32 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
     if (idx == 0x7fffffff) idx = 0;            // fewer experts allowed than asked for
     if (lane == 0) {
       chosen[(long long)t * top + round] = idx;
-      const float s = 1.0f / (1.0f + expf(-z[(long long)t * ldz + idx]));
-      weights[(long long)t * top + round] = v == -INFINITY ? 0.f : s * scale;
+      weights[(long long)t * top + round] = v == -INFINITY ? 0.f : score[idx] * scale;
       choice[idx] = -INFINITY;
     }
     __syncthreads();
+  }
+  if (renormalise && lane == 0) {
+    float total = 0.f;
+    for (int r = 0; r < top; ++r) total += weights[(long long)t * top + r];
+    const float inv = 1.0f / (total + 1e-20f);
+    for (int r = 0; r < top; ++r) weights[(long long)t * top + r] *= inv;
   }
 }
 
 RLIS_API int rlis_moe_route(const float* z, long long ldz, const float* correction, int T, int E,
                             int G, int keep, int top, float scale, int* chosen, float* weights,
+                            int softmax_scores, int group_max, int renormalise,
                             hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && E > 0 && G > 0 && E % G == 0 && keep >= 1 && keep <= G && top >= 1,
                "moe_route: bad sizes E=%d groups=%d keep=%d top=%d", E, G, keep, top);
   RLIS_REQUIRE(top <= keep * (E / G), "moe_route: %d experts asked of %d allowed", top,
                keep * (E / G));
-  RLIS_REQUIRE(E <= 64 * 1024 / 8, "moe_route: too many experts");
+  RLIS_REQUIRE(E <= 64 * 1024 / 16, "moe_route: too many experts");
   if (T == 0) return 0;
-  moe_route_kernel<<<T, 64, (size_t)(E + G) * 4, stream>>>(z, ldz, correction, E, G, keep, top,
-                                                          scale, chosen, weights);
+  moe_route_kernel<<<T, 64, (size_t)(2 * E + G) * 4, stream>>>(
+      z, ldz, correction, E, G, keep, top, scale, chosen, weights, softmax_scores, group_max,
+      renormalise);
   RLIS_LAUNCH_CHECK("moe_route");
   return 0;
 }
@@ -232,7 +267,7 @@ template <typename T, int WAVES, bool ALIGNED>
 __global__ __launch_bounds__(64 * WAVES) void moe_gate_up_kernel(
     const T* __restrict__ x, long long ldx, const T* __restrict__ w_gu,
     const int* __restrict__ sorted, const int* __restrict__ tile_expert, int top, int F, int K,
-    T* __restrict__ hidden) {
+    T* __restrict__ hidden, float limit, float alpha) {
   const int e = tile_expert[blockIdx.x];
   if (e < 0) return;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -255,7 +290,7 @@ __global__ __launch_bounds__(64 * WAVES) void moe_gate_up_kernel(
     for (int i = 0; i < 4; ++i) {
       const int row = row0 + (lane / 16) * 4 + i;
       const float g = acc[b][i], u = acc[b + 2][i];
-      if (f < F) st(hidden + (long long)row * F + f, g / (1.0f + expf(-g)) * u);
+      if (f < F) st(hidden + (long long)row * F + f, gated_unit(g, u, limit, alpha));
     }
   }
 }
@@ -303,7 +338,7 @@ template <typename T, bool ALIGNED>
 __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(
     const T* __restrict__ x, long long ldx, const T* __restrict__ w_gu,
     const int* __restrict__ sorted, const int* __restrict__ tile_expert, int top, int F, int K,
-    T* __restrict__ hidden) {
+    T* __restrict__ hidden, float limit, float alpha) {
   const int e = tile_expert[blockIdx.x];
   if (e < 0) return;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -333,7 +368,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(
       for (int i = 0; i < 4; ++i) {
         const int row = row0 + a * 16 + (lane / 16) * 4 + i;
         const float g = acc[a][b][i], u = acc[a][b + 2][i];
-        if (f < F) st(hidden + (long long)row * F + f, g / (1.0f + expf(-g)) * u);
+        if (f < F) st(hidden + (long long)row * F + f, gated_unit(g, u, limit, alpha));
       }
     }
 }
@@ -390,7 +425,7 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(
     const bf16_t* __restrict__ A, long long lda, const bf16_t* __restrict__ W,
     const int* __restrict__ sorted, const int* __restrict__ tile_expert,
     const float* __restrict__ weights, int top, int N, int K, bf16_t* __restrict__ hidden,
-    float* __restrict__ y) {
+    float* __restrict__ y, float limit, float alpha) {
   constexpr int BM = 128, BK = 64, LDS_STRIDE = BK + 8;
   __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t Bs[BM * LDS_STRIDE];
@@ -484,7 +519,7 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(
       if (GATE_UP) {
         const int f = n0 + wn * 32 + lane % 32;
         const float g = acc[i][0][r], u = acc[i][1][r];
-        if (f < N) hidden[(long long)row * N + f] = f32_to_bf16(g / (1.0f + expf(-g)) * u);
+        if (f < N) hidden[(long long)row * N + f] = f32_to_bf16(gated_unit(g, u, limit, alpha));
       } else {
         const int pair = sorted[row];
         if (pair < 0) continue;
@@ -501,7 +536,8 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(
 RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const void* w_gu,
                               const void* w_d, const int* sorted, const int* tile_expert,
                               const float* weights, int tile_rows, int max_tiles, int top, int F,
-                              int K, void* hidden, float* y, hipStream_t stream) {
+                              int K, void* hidden, float* y, float limit, float alpha,
+                              hipStream_t stream) {
   RLIS_REQUIRE((tile_rows == 16 || tile_rows == 64 || tile_rows == 128) && max_tiles >= 0 &&
                    top > 0 && F > 0 && K > 0,
                "moe_experts: bad sizes");
@@ -516,10 +552,10 @@ RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const voi
     RLIS_REQUIRE(ceil_div(F, 64) <= 65535 && ceil_div(K, 128) <= 65535, "moe_experts: too wide");
     moe_tiles128_kernel<true><<<dim3(max_tiles, ceil_div(F, 64)), 256, 0, stream>>>(
         (const bf16_t*)x, ldx, (const bf16_t*)w_gu, sorted, tile_expert, weights, top, F, K,
-        (bf16_t*)hidden, nullptr);
+        (bf16_t*)hidden, nullptr, limit, alpha);
     moe_tiles128_kernel<false><<<dim3(max_tiles, ceil_div(K, 128)), 256, 0, stream>>>(
         (const bf16_t*)hidden, F, (const bf16_t*)w_d, sorted, tile_expert, weights, top, K, F,
-        nullptr, y);
+        nullptr, y, 0.f, 0.f);
     RLIS_LAUNCH_CHECK("moe_experts");
     return 0;
   }
@@ -529,12 +565,14 @@ RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const voi
   do {                                                                                         \
     if (WAVES == 4) {                                                                          \
       moe_gate_up_rows_kernel<T, AL1><<<dim3(max_tiles, ceil_div(F, 128)), 256, 0, stream>>>(  \
-          (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden);       \
+          (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden, limit, \
+          alpha);                                                                              \
       moe_down_rows_kernel<T, AL2><<<dim3(max_tiles, ceil_div(K, 256)), 256, 0, stream>>>(     \
           (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);             \
     } else {                                                                                   \
       moe_gate_up_kernel<T, WAVES, AL1><<<g1, 64 * WAVES, 0, stream>>>(                        \
-          (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden);       \
+          (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden, limit, \
+          alpha);                                                                              \
       moe_down_kernel<T, WAVES, AL2><<<g2, 64 * WAVES, 0, stream>>>(                           \
           (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);             \
     }                                                                                          \

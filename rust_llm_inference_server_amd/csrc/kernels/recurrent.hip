@@ -76,7 +76,10 @@ __global__ void tail_update_kernel(float* __restrict__ state, long long state_st
 }
 
 // ------------------------------------------- short causal convolution + SiLU (+ unit norm)
-// y[t][c] = silu(bias[c] + sum_j taps[c][j] * x[t - (K - 1) + j][c]) (bias optional); rows in front of the step come from
+// y[t][c] = act(bias[c] + sum_j taps[c][j] * x[t - (K - 1) + j][c]) (bias optional; act is SiLU,
+// or nothing with activation 0); channels from blend_from on are then mixed with another
+// tensor's rows of the same tokens, y <- (1 - blend_weight) y + blend_weight * blend[t][c -
+// blend_from] (blend null: no mixing); rows in front of the step come from
 // the tail, rows in front of the sequence are the tail's zeros.  Channels [0, unit_channels)
 // are then made unit vectors in groups of unit_group (x / sqrt(sum x^2 + unit_eps)) and those
 // below scaled_channels multiplied by `scale`; the other channels are cut into groups of
@@ -92,7 +95,8 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     const float* __restrict__ state, long long state_stride,
     const int* __restrict__ seq_of_token, const int* __restrict__ cu,
     const int* __restrict__ slots, int unit_channels, int unit_group, int scaled_channels,
-    float scale, float unit_eps, int rest_group, int groups) {
+    float scale, float unit_eps, int rest_group, int groups, int activation,
+    const TO* __restrict__ blend, long long ld_blend, int blend_from, float blend_weight) {
   const int t = blockIdx.x;
   const int lane = threadIdx.x % kWave;
   const int g = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -128,7 +132,11 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
         const float from_tail = R > 0 ? tail[(long long)(here ? 0 : R - (back - rel)) * C + c] : 0.f;
         acc += taps[(long long)c * K + j] * (here ? from_step : from_tail);
       }
-      y[v] = off < width ? siluf_(acc) : 0.f;
+      if (activation) acc = siluf_(acc);
+      if (blend && c >= blend_from)
+        acc = (1.0f - blend_weight) * acc +
+              blend_weight * ld(blend + (long long)t * ld_blend + (c - blend_from));
+      y[v] = off < width ? acc : 0.f;
       ss += y[v] * y[v];
     }
   }
@@ -778,12 +786,14 @@ __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
 }
 
 // --------------------------------------------------- per-head RMS norm, weight and gate
-// y[t][h][j] = o / sqrt(mean_j o^2 + eps) * weight[h * weight_stride + j] * silu(gate[t][h][j]).
-// One wave per (token, head).
+// y[t][h][j] = o / sqrt(mean_j o^2 + eps) * weight[h * weight_stride + j] * silu(gate[t][h][j])
+// (with sigmoid_gate: * sigmoid(gate[t][h][j])).  One wave per (token, head); one head of
+// heads * dv channels is the norm over the heads together.
 template <typename TG, typename TO>
 __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(
     TO* __restrict__ out, const float* __restrict__ o, const float* __restrict__ weight,
-    int weight_stride, const TG* __restrict__ gate, long long ldg, int heads, int dv, float eps) {
+    int weight_stride, const TG* __restrict__ gate, long long ldg, int heads, int dv, float eps,
+    int sigmoid_gate) {
   const int t = blockIdx.x, h = blockIdx.y;
   const float* row = o + ((long long)t * heads + h) * dv;
   float ss = 0.f;
@@ -793,7 +803,8 @@ __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(
   for (int j = threadIdx.x; j < dv; j += kWave) {
     const float g = ld(gate + (long long)t * ldg + h * dv + j);
     st(out + ((long long)t * heads + h) * dv + j,
-       row[j] * inv * weight[h * weight_stride + j] * siluf_(g));
+       row[j] * inv * weight[h * weight_stride + j] *
+           (sigmoid_gate ? 1.0f / (1.0f + expf(-g)) : siluf_(g)));
   }
 }
 
@@ -859,8 +870,12 @@ RLIS_API int rlis_causal_conv(void* out, int out_dtype, const float* x, long lon
                               long long state_stride,
                               const int* seq_of_token, const int* cu, const int* slots, int T,
                               int unit_channels, int unit_group, int scaled_channels, float scale,
-                              float unit_eps, int rest_group, hipStream_t stream) {
+                              float unit_eps, int rest_group, int activation, const void* blend,
+                              long long ld_blend, int blend_from, float blend_weight,
+                              hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && C > 0 && K >= 1 && K <= 16, "causal_conv: bad sizes T=%d C=%d taps=%d", T, C, K);
+  RLIS_REQUIRE(!blend || (blend_from >= 0 && blend_from < C && ld_blend >= C - blend_from),
+               "causal_conv: the rows to mix in do not cover channels %d to %d", blend_from, C);
   RLIS_REQUIRE(ldx >= C && state_stride >= (long long)C * (K - 1), "causal_conv: strides too short");
   RLIS_REQUIRE(unit_channels >= 0 && unit_channels <= C && scaled_channels <= unit_channels,
                "causal_conv: bad channel ranges");
@@ -878,7 +893,8 @@ RLIS_API int rlis_causal_conv(void* out, int out_dtype, const float* x, long lon
   causal_conv_kernel<TO><<<dim3(T, ceil_div(groups, 4)), 256, 0, stream>>>(                    \
       (TO*)out, x, ldx, taps, bias, C, K, state, state_stride, seq_of_token, cu, slots,        \
       unit_channels, unit_group, scaled_channels, scale, unit_eps,                             \
-      rest_group > 0 ? rest_group : 1, groups)
+      rest_group > 0 ? rest_group : 1, groups, activation, (const TO*)blend, ld_blend,         \
+      blend_from, blend_weight)
   if (out_dtype == RLIS_F32) LAUNCH(float);
   else if (out_dtype == RLIS_BF16) LAUNCH(bf16_t);
   else RLIS_REQUIRE(false, "causal_conv: unknown dtype %d", out_dtype);
@@ -973,7 +989,7 @@ RLIS_API int rlis_decay_scan(float* out, const float* r, const float* k, const f
 RLIS_API int rlis_head_norm_gate(void* out, int out_dtype, const float* o, const float* weight,
                                  int weight_stride, const void* gate, int gate_dtype,
                                  long long ldg, int T, int heads, int dv, float eps,
-                                 hipStream_t stream) {
+                                 int sigmoid_gate, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && heads > 0 && dv > 0 && heads <= 65535,
                "head_norm_gate: bad sizes T=%d heads=%d dv=%d", T, heads, dv);
   RLIS_REQUIRE(weight_stride == 0 || weight_stride == dv, "head_norm_gate: bad weight stride");
@@ -983,7 +999,8 @@ RLIS_API int rlis_head_norm_gate(void* out, int out_dtype, const float* o, const
 #define CASE(k_, TG, TO)                                                                     \
   case k_:                                                                                   \
     head_norm_gate_kernel<TG, TO><<<grid, kWave, 0, stream>>>(                               \
-        (TO*)out, o, weight, weight_stride, (const TG*)gate, ldg, heads, dv, eps);           \
+        (TO*)out, o, weight, weight_stride, (const TG*)gate, ldg, heads, dv, eps,            \
+        sigmoid_gate);                                                                       \
     break;
   switch (key) {
     CASE(0, float, float)

@@ -75,6 +75,10 @@ class StepContext:
     # stays where it is).
     buffer: Optional[torch.Tensor] = None
     over: Optional[Callable[[torch.Tensor], "StepContext"]] = None
+    # What a layer's parts hand on to the parts of later layers within one forward pass, by
+    # name (rows of the step's own tokens, e.g. the values that later layers mix into theirs);
+    # emptied when a pass begins.
+    carried: Dict[str, Any] = field(default_factory=dict)
 
 
 class MetadataBuffer:

@@ -178,7 +178,12 @@ class Model:
     def forward(self, step: Any, pools: Any) -> torch.Tensor:
         """Logits float32 ``(R, V)`` at ``step.logit_rows``; K, V and state of the step's
         tokens are left in ``pools``."""
-        stream = ResidualStream(self.embedding.forward(step.ids), self.act_dtype)
+        rows = self.embedding.position_rows
+        if rows is not None and step.max_context > rows:
+            raise ValueError(f"sequence of {step.max_context} positions exceeds the model's "
+                             f"{rows} learned positions")
+        step.carried.clear()
+        stream = ResidualStream(self.embedding.forward(step.ids, step.positions), self.act_dtype)
         for i, run in enumerate(self.runs):
             self.layers[run.layer].forward(stream, step, pools.binding(self.bindings[i]))
         if step.num_logit_rows == 0:

@@ -172,16 +172,60 @@ def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> int:
 
 
 # --------------------------------------------------------------------------- rows
-def embed(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
-    """Rows ``table[ids] * scale`` as the float32 residual stream ``(T, H)``."""
+def embed(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0,
+          learned: Optional[torch.Tensor] = None,
+          positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rows ``table[ids] * scale`` as the float32 residual stream ``(T, H)``; with ``learned``
+    (a table ``(max positions, H)`` of the embedding table's dtype) plus
+    ``learned[positions]``, added as it is."""
     _check(table, "embed table", ndim=2)
     T, (V, H) = ids.numel(), table.shape
     if not table.is_contiguous():
         raise KernelError("embed table must be contiguous")
+    learned_ptr = pos_ptr = None
+    if learned is not None:
+        _check(learned, "learned positions", table.dtype, 2)
+        if learned.shape[1] != H or not learned.is_contiguous() or positions is None:
+            raise KernelError("embed: learned position vectors must be contiguous rows of the "
+                              "table's width, and need the tokens' positions")
+        learned_ptr, pos_ptr = learned.data_ptr(), _i32(positions, "positions", T)
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     lib.call("rlis_embed", out.data_ptr(), table.data_ptr(), _dt(table), _i32(ids, "ids", T),
-             T, H, float(scale), lib.stream_ptr())
+             T, H, float(scale), learned_ptr, pos_ptr, lib.stream_ptr())
     return out
+
+
+def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
+    """``0.5 x (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3)))``, float32 arithmetic."""
+    _check(x, "gelu_tanh")
+    if not x.is_contiguous():
+        raise KernelError("gelu_tanh: tensor must be contiguous")
+    out = torch.empty_like(x)
+    lib.call("rlis_gelu_tanh", out.data_ptr(), x.data_ptr(), _dt(x), x.numel(), lib.stream_ptr())
+    return out
+
+
+def depth_mix_(x: torch.Tensor, delta: torch.Tensor, history: torch.Tensor, count: int,
+               weights: torch.Tensor, save_input: bool = False) -> None:
+    """``history (slots, T, W)`` float32 holds the embedding output and every layer's result so
+    far.  This layer's result ``x + delta`` becomes source ``count - 1``, and ``x`` becomes
+    ``sum_j weights[j] * history[j]`` over the ``count`` sources, in place, in float32.
+    ``save_input`` (the first layer, ``count`` 2): ``x`` itself is stored as source 0 first."""
+    _check(x, "depth_mix x", torch.float32, 2)
+    _check(delta, "depth_mix delta", torch.float32, 2)
+    _check(history, "depth_mix history", torch.float32, 3)
+    _check(weights, "depth_mix weights", ndim=1)
+    if delta.shape != x.shape or tuple(history.shape[1:]) != tuple(x.shape) \
+            or not (x.is_contiguous() and delta.is_contiguous() and history.is_contiguous()):
+        raise KernelError("depth_mix: x, delta and the slabs of history must be contiguous and "
+                          "of one shape")
+    if not 2 <= count <= history.shape[0] or weights.numel() != count \
+            or not weights.is_contiguous():
+        raise KernelError(f"depth_mix: {count} sources, {weights.numel()} weights, "
+                          f"{history.shape[0]} slabs")
+    lib.call("rlis_depth_mix", x.data_ptr(), delta.data_ptr(), history.data_ptr(), x.numel(),
+             int(count), weights.data_ptr(), _dt(weights), int(bool(save_input)),
+             lib.stream_ptr())
 
 
 def _delta_parts(resid: torch.Tensor, delta: torch.Tensor, what: str) -> int:
@@ -793,29 +837,39 @@ def _prefill_mfma_ok(qkv: torch.Tensor, d: int, page_size: int) -> bool:
             and AttentionPlanner.pages_fit(page_size) and qkv.stride(0) % 8 == 0)
 
 
+# Whether scores with a scale per head or a cap take the matrix-core kernels (False: the
+# vector-unit kernels, for tests that hold the two against each other).
+SHAPED_SCORES_MATRIX = False
+
+
 def attention_planner(num_heads: int, num_kv_heads: int, head_dim: int,
-                      dtype: torch.dtype, biased: bool = False) -> AttentionPlanner:
+                      dtype: torch.dtype, biased: bool = False,
+                      shaped: bool = False) -> AttentionPlanner:
     """The planner a mixer that calls ``paged_attention`` / ``rope_attention`` names as its
     ``step_planner()``; ``biased``: it will pass ``bias_slopes`` (the matrix-core kernels take
-    them too, so the plan is the same)."""
+    them too, so the plan is the same); ``shaped``: it will pass ``head_scales`` or a
+    ``softcap``."""
     return AttentionPlanner(num_heads, num_kv_heads, head_dim,
-                            matrix=dtype == torch.bfloat16,
+                            matrix=dtype == torch.bfloat16
+                            and (not shaped or SHAPED_SCORES_MATRIX),
                             singles_apart=SPLIT_MIXED_ATTENTION and DECODE_ATTENTION != "vector")
 
 
 def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
-                      force: Optional[str], biased: bool = False):
+                      force: Optional[str], biased: bool = False, shaped: bool = False):
     """(kind, matrix_decode): which attention kernel a batch takes.  A bias on the scores
-    changes nothing here: every kernel takes one."""
+    changes nothing here: every kernel takes one.  ``shaped`` (a scale per head, a cap on the
+    scores): the matrix-core kernels take it when ``SHAPED_SCORES_MATRIX`` says so."""
     kind = force or FORCE_ATTENTION
+    matrix = not shaped or SHAPED_SCORES_MATRIX
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
-        elif _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode:
+        elif matrix and _prefill_mfma_ok(qkv, d, page_size) and not step.all_decode:
             kind = "prefill"
         else:
             kind = "generic"
-    mfma = kind == "decode" and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
+    mfma = kind == "decode" and matrix and _decode_mfma_ok(qkv, nh, nkv, d, page_size)
     return kind, mfma
 
 
@@ -838,8 +892,11 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                    window: Optional[int] = None, write_kv: bool = True,
                    plan: Optional[StepPlan] = None, interleaved: bool = False,
                    bias_slopes: Optional[torch.Tensor] = None,
-                   counters: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``rope_kv_write`` followed by ``paged_attention``.  A decode batch that takes the
+                   counters: Optional[torch.Tensor] = None,
+                   head_scales: Optional[torch.Tensor] = None,
+                   softcap: float = 0.0) -> torch.Tensor:
+    """``rope_kv_write`` followed by ``paged_attention`` (``head_scales`` and ``softcap`` as
+    there).  A decode batch that takes the
     matrix-core decode kernel does both in that kernel when the whole head is rotated
     (rotate-half) and is 64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left
     unrotated.  Under the same conditions a batch with portions of prompts leaves the queries
@@ -849,7 +906,9 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     and ``paged_attention``."""
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     _rows_contig(qkv, "qkv")
-    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None, bias_slopes is not None)
+    shaped = head_scales is not None or softcap > 0
+    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None, bias_slopes is not None,
+                                   shaped)
     fusable = cos is None or (2 * cos.shape[1] == d and d in (64, 128, 256) and not interleaved)
     whole_rows = qkv.shape[1] == (nh + 2 * nkv) * d
     if cos is not None and fusable and whole_rows and (mfma or kind == "prefill"):
@@ -862,7 +921,8 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
             raise KernelError("rope_attention: a cache write needs slots")
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
-                               bias_slopes=bias_slopes,
+                               bias_slopes=bias_slopes, head_scales=head_scales,
+                               softcap=softcap,
                                rope=(cos, sin, positions, slots if write_kv else None))
     if (kind == "prefill" and cos is not None and fusable and FUSE_ROPE_PREFILL and whole_rows
             and (_decode_mfma_ok(qkv, nh, nkv, d, page_size)
@@ -871,11 +931,13 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                       write_kv=write_kv, rotate_q=False)
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
-                               bias_slopes=bias_slopes, rope=(cos, sin, positions, None))
+                               bias_slopes=bias_slopes, head_scales=head_scales,
+                               softcap=softcap, rope=(cos, sin, positions, None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
                   write_kv=write_kv, interleaved=interleaved)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
-                           scale, window, plan=plan, bias_slopes=bias_slopes, counters=counters)
+                           scale, window, plan=plan, bias_slopes=bias_slopes, counters=counters,
+                           head_scales=head_scales, softcap=softcap)
 
 
 def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -884,7 +946,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                     window: Optional[int] = None, force: Optional[str] = None,
                     rope: Optional[tuple] = None, plan: Optional[StepPlan] = None,
                     bias_slopes: Optional[torch.Tensor] = None,
-                    counters: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    counters: Optional[torch.Tensor] = None,
+                    head_scales: Optional[torch.Tensor] = None,
+                    softcap: float = 0.0) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
 
     ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
@@ -898,6 +962,9 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     ``bias_slopes`` (float32, one per query head; the reference has no such thing): the score of
     key position ``u`` for a query at position ``p`` gets ``slope * (u - p)`` added before the
     softmax; every kernel takes it (the matrix-core ones in a form of their own).
+    ``head_scales`` (float32, one per query head): the head's scores are multiplied by its
+    number on top of ``scale``; ``softcap`` c > 0: the scaled score becomes ``c * tanh(score /
+    c)`` before bias and softmax.  Both are float32 arithmetic in every kernel.
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
     to rotate and store the step's tokens itself; with portions of prompts in the batch
@@ -936,7 +1003,18 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         if bias_slopes.numel() != nh or not bias_slopes.is_contiguous():
             raise KernelError(f"attention: {bias_slopes.numel()} bias slopes for {nh} heads")
         slopes_ptr = bias_slopes.data_ptr()
-    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force, slopes_ptr is not None)
+    scales_ptr = None
+    if head_scales is not None:
+        _check(head_scales, "head_scales", torch.float32, 1)
+        if head_scales.numel() != nh or not head_scales.is_contiguous():
+            raise KernelError(f"attention: {head_scales.numel()} head scales for {nh} heads")
+        scales_ptr = head_scales.data_ptr()
+    softcap = float(softcap or 0.0)
+    if softcap < 0:
+        raise KernelError("attention: the cap of the scores must be positive (0: none)")
+    shaped = scales_ptr is not None or softcap > 0
+    kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force, slopes_ptr is not None,
+                                   shaped)
     if rope is not None and not (mfma or (kind == "prefill" and rope[3] is None
                                           and rope[0] is not None)):
         raise KernelError("attention: only the matrix-core kernels rotate, and only the decode "
@@ -945,7 +1023,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         lib.call("rlis_attn_generic", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(), nh * d,
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
                  _i32(step.seq_of_token, "seq_of_token", T), _i32(step.positions, "positions", T),
-                 T, nh, nkv, d, page_size, float(scale), win, slopes_ptr, stream)
+                 T, nh, nkv, d, page_size, float(scale), win, slopes_ptr, scales_ptr, softcap,
+                 stream)
         return out
     if kind not in ("decode", "prefill"):
         raise KernelError(f"attention: unknown kernel '{kind}'")
@@ -998,7 +1077,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), None,
                      S, nh, nkv, d, page_size, float(scale), win, depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, slopes_ptr, stream)
+                     ap.DECODE_MAX_PARTS, slopes_ptr, scales_ptr, softcap, stream)
 
     if kind == "decode":
         if not step.all_decode:
@@ -1087,8 +1166,8 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
     return out
 
 
-from .recurrent import (causal_conv, decay_scan, delta_scan, head_norm_gate,  # noqa: E402,F401
-                        selective_scan, shift_mix, tail_update)
+from .recurrent import (causal_conv, decay_attention, decay_scan, delta_scan,  # noqa: E402,F401
+                        head_norm_gate, selective_scan, shift_mix, tail_update)
 from .latent import (head_linear, latent_attention, latent_mfma_ok, latent_write,  # noqa: E402,F401
                      sigmoid_gate_)
 from .routed import routed_units, route, router_logits  # noqa: E402,F401

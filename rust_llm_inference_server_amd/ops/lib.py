@@ -17,7 +17,10 @@ _LIB: Optional[ctypes.CDLL] = None
 P, I, L, F = c_void_p, c_int, c_longlong, c_float
 
 _SIGNATURES = {
-    "rlis_embed": [P, P, I, P, I, I, F, P],
+    "rlis_embed": [P, P, I, P, I, I, F, P, P, P],
+    "rlis_gelu_tanh": [P, P, I, L, P],
+    "rlis_depth_mix": [P, P, P, L, I, P, I, I, P],
+    "rlis_decay_attention_scan": [P, P, L, P, L, P, L, I, P, P, L, P, P, I, I, I, I, I, I, P],
     "rlis_add_residual": [P, P, I, L, I, I, F, P],
     "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
     "rlis_swiglu": [P, P, I, I, I, P],
@@ -26,7 +29,7 @@ _SIGNATURES = {
     "rlis_soft_cap": [P, I, L, F, P],
     "rlis_shift_mix": [P, P, I, P, P, L, P, P, P, I, I, I, P],
     "rlis_tail_update": [P, L, P, I, L, I, I, P, P, I, P],
-    "rlis_causal_conv": [P, I, P, L, P, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, P],
+    "rlis_causal_conv": [P, I, P, L, P, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, I, P, L, I, F, P],
     "rlis_selective_scan": [P, I, L, P, L, P, L, P, P, P, L, P, L, P, P, P, L, P, P, I, I, I, I, I, I,
                             P, P, P],
     "rlis_add_layernorm": [P, P, I, P, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
@@ -37,13 +40,13 @@ _SIGNATURES = {
     "rlis_latent_attention": [P, I, L, P, L, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_sigmoid_gate": [P, L, P, L, I, I, I, P],
     "rlis_moe_router_logits": [P, P, P, F, P, I, P, I, I, I, P],
-    "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, P],
+    "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, I, I, I, P],
     "rlis_moe_sort": [P, I, I, I, I, P, P, P],
-    "rlis_moe_experts": [P, I, L, P, P, P, P, P, I, I, I, I, I, P, P, P],
+    "rlis_moe_experts": [P, I, L, P, P, P, P, P, I, I, I, I, I, P, P, F, F, P],
     "rlis_moe_combine": [P, P, P, I, I, I, I, P],
     "rlis_delta_scan": [P, L, P, P, P, L, P, P, L, P, P, P, L, P, P, I, I, I, I, I, I, P],
     "rlis_decay_scan": [P, P, P, P, P, L, P, P, P, L, P, P, I, I, I, I, P],
-    "rlis_head_norm_gate": [P, I, P, P, I, P, I, L, I, I, I, F, P],
+    "rlis_head_norm_gate": [P, I, P, P, I, P, I, L, I, I, I, F, I, P],
     "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
     "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],
     "rlis_gemm_plain": [P, I, P, I, P, I, I, I, I, L, L, L, P],
@@ -55,8 +58,8 @@ _SIGNATURES = {
     "rlis_gemm_bf16_stream_join": [P, P, I, I, I, L, L, P, P, P, I, I, P, P, I, P],
     "rlis_gemm_bf16_stream_scaled": [P, P, P, I, I, I, I, L, L, L, I, P, I, I, F, P],
     "rlis_norm_linear_bf16": [P, P, I, I, L, I, P, I, F, P, P, P, P, I, I, I, I, L, L, I, P],
-    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
-    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P],
+    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P, F, P],
+    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P, F, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, I, I, I,
                               P, P, I, P, P, L, L, P, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,

@@ -110,10 +110,15 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor,
                 unit_channels: int = 0, unit_group: int = 0, scaled_channels: int = 0,
                 scale: float = 1.0, unit_eps: float = 0.0, rest_group: int = 256,
                 bias: Optional[torch.Tensor] = None,
-                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                out_dtype: torch.dtype = torch.float32, activation: bool = True,
+                blend: Optional[torch.Tensor] = None, blend_from: int = 0,
+                blend_weight: float = 0.0) -> torch.Tensor:
     """``silu`` of the causal convolution over time of the first ``C`` columns of ``x`` (float32)
     with ``taps (C, K)`` (the last column multiplies the current row; the ``K - 1`` rows in
-    front of the step come from ``state``), plus ``bias (C)`` under the ``silu`` when given.  Channels below ``unit_channels`` are then made
+    front of the step come from ``state``), plus ``bias (C)`` under the ``silu`` when given;
+    without ``activation`` the convolution as it is.  With ``blend`` (rows of the same tokens in
+    ``out_dtype``, ``C - blend_from`` columns) the channels from ``blend_from`` on become
+    ``(1 - blend_weight) * y + blend_weight * blend``.  Channels below ``unit_channels`` are then made
     unit vectors in groups of ``unit_group``: ``y / sqrt(sum y^2 + unit_eps)``, those below
     ``scaled_channels`` times ``scale``.  Returns ``(T, C)`` in ``out_dtype`` (float32 arithmetic)."""
     ldx = _rows(x, "causal_conv x", torch.float32)
@@ -124,12 +129,20 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor,
     T = x.shape[0]
     stride = _state(state, C * (K - 1), "causal_conv")
     out = torch.empty((T, C), dtype=out_dtype, device=x.device)
+    blend_ptr, ld_blend = None, 0
+    if blend is not None:
+        ld_blend = _rows(blend, "causal_conv blend", out_dtype)
+        if blend.shape[0] != T or blend.shape[1] != C - blend_from or not 0 <= blend_from < C:
+            raise KernelError(f"causal_conv: rows to mix in of shape {tuple(blend.shape)} for "
+                              f"channels {blend_from} to {C} of {T} tokens")
+        blend_ptr = blend.data_ptr()
     lib.call("rlis_causal_conv", out.data_ptr(), _DT[out_dtype], x.data_ptr(), ldx,
              taps.data_ptr(), None if bias is None else _vec(bias, C, "causal_conv bias"), C, K,
              state.data_ptr(), stride, _meta(seq_of_token, T, "seq_of_token"),
              _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), T,
              int(unit_channels), int(unit_group), int(scaled_channels), float(scale),
-             float(unit_eps), int(rest_group), lib.stream_ptr())
+             float(unit_eps), int(rest_group), int(bool(activation)), blend_ptr, ld_blend,
+             int(blend_from), float(blend_weight), lib.stream_ptr())
     return out
 
 
@@ -194,9 +207,10 @@ def decay_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tenso
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, heads: int, dv: int,
-                   eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+                   eps: float, out_dtype: torch.dtype, sigmoid_gate: bool = False) -> torch.Tensor:
     """``o / sqrt(mean o^2 + eps)`` per head, times ``weight`` (``heads * dv`` values, or ``dv``
-    shared by the heads), times ``silu(gate)``.  ``o`` contiguous float32 ``(T, heads * dv)``,
+    shared by the heads), times ``silu(gate)`` (``sigmoid_gate``: times ``sigmoid(gate)``).  One
+    head of all the channels is the norm over the heads together.  ``o`` contiguous float32 ``(T, heads * dv)``,
     ``gate`` of that shape with contiguous rows."""
     T = o.shape[0]
     if not o.is_cuda or o.dtype != torch.float32 or o.shape != (T, heads * dv) \
@@ -216,7 +230,34 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, he
     out = torch.empty((T, heads * dv), dtype=out_dtype, device=o.device)
     lib.call("rlis_head_norm_gate", out.data_ptr(), _DT[out_dtype], o.data_ptr(),
              weight.data_ptr(), wstride, gate.data_ptr(), _dt(gate), ldg, T, heads, dv, float(eps),
-             lib.stream_ptr())
+             int(bool(sigmoid_gate)), lib.stream_ptr())
+    return out
+
+
+def decay_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,
+                    state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
+                    heads: int, dim: int, vdim: int, activation: bool = True) -> torch.Tensor:
+    """Linear attention with a fixed decay per head: ``S <- decay[h] S + k v^T``, ``o = S^T q``
+    (the token's own key and value are in what its query reads).  ``q``, ``k`` ``(T, heads *
+    dim)`` and ``v`` ``(T, heads * vdim)`` are the raw projections of one dtype, with row
+    strides; they pass SiLU in float32 on the way in (``activation``).  ``state``: per slot
+    ``heads * vdim * dim`` float32, left as after each sequence's last token.  Returns
+    ``(T, heads * vdim)`` float32."""
+    T = q.shape[0]
+    ldq, ldk, ldv = _rows(q, "decay_attention q"), _rows(k, "decay_attention k"), \
+        _rows(v, "decay_attention v")
+    if q.dtype != k.dtype or q.dtype != v.dtype or k.shape[0] != T or v.shape[0] != T \
+            or q.shape[1] != heads * dim or k.shape[1] != heads * dim \
+            or v.shape[1] != heads * vdim:
+        raise KernelError("decay_attention: q, k (T, heads * dim) and v (T, heads * vdim) of one "
+                          "dtype")
+    stride = _state(state, heads * vdim * dim, "decay_attention")
+    out = torch.empty((T, heads * vdim), dtype=torch.float32, device=q.device)
+    lib.call("rlis_decay_attention_scan", out.data_ptr(), q.data_ptr(), ldq, k.data_ptr(), ldk,
+             v.data_ptr(), ldv, _dt(q), _vec(decay, heads, "decay_attention decay"),
+             state.data_ptr(), stride, _meta(cu, num_seqs + 1, "cu"),
+             _meta(slots, num_seqs, "slots"), num_seqs, T, heads, dim, vdim,
+             int(bool(activation)), lib.stream_ptr())
     return out
 
 

@@ -47,36 +47,46 @@ def router_logits(resid: torch.Tensor, norm_weight: torch.Tensor, norm_bias: tor
     return z
 
 
-def route(logits: torch.Tensor, correction: torch.Tensor, groups: int, keep: int, top: int,
-          scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
-    """From router logits ``(T, E)`` float32: scores ``s = sigmoid(logits)``, choice scores
-    ``s + correction``; experts stand in ``groups`` equal groups of neighbours, a group's score
-    is the sum of its two largest choice scores, and only experts of the ``keep`` best groups
-    can be chosen; the ``top`` largest choice scores win.  Returns the chosen experts
-    ``(T, top)`` int32 and their weights ``s * scale`` ``(T, top)`` float32."""
+def route(logits: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int,
+          top: int, scale: float, scores: str = "sigmoid", group_score: str = "top2",
+          renormalise: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """From router logits ``(T, E)`` float32: scores ``s = sigmoid(logits)`` (``scores``
+    "softmax": their softmax over all experts), choice scores ``s + correction`` (None: no
+    correction); experts stand in ``groups`` equal groups of neighbours, a group's score
+    is the sum of its two largest choice scores (``group_score`` "max": the largest), and only
+    experts of the ``keep`` best groups can be chosen; the ``top`` largest choice scores win.
+    Returns the chosen experts ``(T, top)`` int32 and their weights ``(T, top)`` float32:
+    ``s * scale``, with ``renormalise`` divided by their sum + 1e-20."""
     if not logits.is_cuda or logits.dtype != torch.float32 or logits.dim() != 2 \
             or (logits.shape[1] > 1 and logits.stride(1) != 1):
         raise KernelError("route: the logits must be float32 (T, E) on the GPU")
     T, E = logits.shape
-    if correction.dtype != torch.float32 or correction.numel() != E \
-            or not correction.is_contiguous():
+    if correction is not None and (correction.dtype != torch.float32 or correction.numel() != E
+                                   or not correction.is_contiguous()):
         raise KernelError(f"route: the correction must be {E} float32 values")
+    if scores not in ("sigmoid", "softmax") or group_score not in ("top2", "max"):
+        raise KernelError(f"route: unknown scores '{scores}' or group score '{group_score}'")
     ldz = logits.stride(0) if T > 1 else max(logits.stride(0), E)
     chosen = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
-    lib.call("rlis_moe_route", logits.data_ptr(), ldz, correction.data_ptr(), T, E, int(groups),
+    lib.call("rlis_moe_route", logits.data_ptr(), ldz,
+             None if correction is None else correction.data_ptr(), T, E, int(groups),
              int(keep), int(top), float(scale), chosen.data_ptr(), weights.data_ptr(),
+             int(scores == "softmax"), int(group_score == "max"), int(bool(renormalise)),
              lib.stream_ptr())
     return chosen, weights
 
 
 def routed_units(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
                  chosen: torch.Tensor, weights: torch.Tensor,
-                 addend: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 addend: Optional[torch.Tensor] = None, limit: float = 0.0,
+                 alpha: float = 1.0) -> torch.Tensor:
     """``out[t] = sum_k weights[t, k] * unit(chosen[t, k], x[t])  (+ addend[t])`` in float32,
     where unit ``e`` is ``Wd[e] (silu(Wg[e] x) * (Wu[e] x))`` with ``w_gate_up (E, 2 F, W)``
     (an expert's gate rows in front of its up rows) and ``w_down (E, W, F)``, both in the dtype
-    of ``x (T, W)``.  A token's units are added in the order of its choices."""
+    of ``x (T, W)``.  A token's units are added in the order of its choices.  ``limit`` > 0: the
+    units are of the bounded kind, ``Wd[e] (g sigmoid(alpha g) (u + 1))`` with
+    ``g = min(Wg[e] x, limit)`` and ``u = clamp(Wu[e] x, -limit, limit)``."""
     if not x.is_cuda or x.dim() != 2 or x.dtype not in _DT or (x.shape[1] > 1 and x.stride(1) != 1):
         raise KernelError("routed_units: x must be (T, W) on the GPU with contiguous rows")
     T, W = x.shape
@@ -109,7 +119,8 @@ def routed_units(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
     ldx = x.stride(0) if T > 1 else max(x.stride(0), W)
     lib.call("rlis_moe_experts", x.data_ptr(), _DT[x.dtype], ldx, w_gate_up.data_ptr(),
              w_down.data_ptr(), order.data_ptr(), tile_expert.data_ptr(), weights.data_ptr(),
-             rows, tiles, top, F, W, hidden.data_ptr(), y.data_ptr(), lib.stream_ptr())
+             rows, tiles, top, F, W, hidden.data_ptr(), y.data_ptr(), float(limit), float(alpha),
+             lib.stream_ptr())
     if addend is not None and (tuple(addend.shape) != (T, W) or not addend.is_contiguous()
                                or addend.dtype not in _DT):
         raise KernelError("routed_units: the addend must be a contiguous (T, W) tensor")

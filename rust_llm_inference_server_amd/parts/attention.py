@@ -14,8 +14,8 @@ from typing import Any, Dict, List, Optional
 import torch
 
 from .. import ops
-from .base import (BuildContext, CacheBinding, CacheRequest, Mixer, PartSpec, TensorSpec, join,
-                   project, register)
+from .base import (BuildContext, CacheBinding, CacheRequest, Mixer, NormedInput, PartSpec,
+                   TensorSpec, join, project, register)
 from .rope import shared_position
 
 
@@ -25,7 +25,21 @@ class PagedAttention(Mixer):
     ``window`` (None: all earlier positions), ``position`` (a PartSpec); optional ``value_dim``
     (size of a value head when it differs from ``head_dim``, the size of a query and key head)
     and ``names`` (the tensors of q, k, v and o under the prefix; default ``q_proj.weight`` and
-    so on).
+    so on).  Further options, none of which the reference's Llama has:
+
+    * ``conv`` (taps K): a short causal convolution over time on every channel of q, k and v,
+      directly behind the projection and in front of the rotation, no bias, no activation:
+      ``y_t = sum_j w[:, j] u_(t - K + 1 + j)`` with zeros in front of the sequence; tensors
+      ``<q|k|v name>.conv`` (channels, K).  The last K - 1 projected rows of a request live in
+      its state slot (float32); the products' results are float32 and the convolution is
+      float32 arithmetic.
+    * ``head_scales``: the name (under the prefix) of a tensor with one number per query head
+      that multiplies the head's scores on top of ``scale``.
+    * ``softcap`` c: the scaled score becomes ``c tanh(score / c)`` in front of the softmax.
+    * ``value_mix``: ``{"name": tensor under the prefix, "key": a name, "source": bool}``.
+      The source layer hands its values (behind the convolution) on to the later layers of the
+      step under ``key``; every other layer with that key replaces its values by
+      ``(1 - w) v + w v_source`` (``w`` the tensor's one number) before they are cached.
 
     With ``value_dim != head_dim`` the kernels run at one head size ``D``, the larger of the two
     rounded up to a multiple of 16: the rows of the narrower projection's weight are padded
@@ -54,8 +68,18 @@ class PagedAttention(Mixer):
                                              "head_dim"))
         dv = params.get("value_dim") or d
         n = cls._names(params, prefix)
-        return [TensorSpec(n["q"], (nh * d, H)), TensorSpec(n["k"], (nkv * d, H)),
-                TensorSpec(n["v"], (nkv * dv, H)), TensorSpec(n["o"], (H, nh * dv))]
+        out = [TensorSpec(n["q"], (nh * d, H)), TensorSpec(n["k"], (nkv * d, H)),
+               TensorSpec(n["v"], (nkv * dv, H)), TensorSpec(n["o"], (H, nh * dv))]
+        taps = params.get("conv")
+        if taps:
+            out += [TensorSpec(n[c] + ".conv", (rows, int(taps)), std=0.3)
+                    for c, rows in (("q", nh * d), ("k", nkv * d), ("v", nkv * dv))]
+        if params.get("head_scales"):
+            out.append(TensorSpec(join(prefix, params["head_scales"]), (nh,), init="ones_normal",
+                                  std=0.2))
+        if params.get("value_mix"):
+            out.append(TensorSpec(join(prefix, params["value_mix"]["name"]), (), std=0.3))
+        return out
 
     @staticmethod
     def _pad_heads(w: torch.Tensor, heads: int, size: int, to: int, rows: bool) -> torch.Tensor:
@@ -79,6 +103,7 @@ class PagedAttention(Mixer):
         v_dim = int(params.get("value_dim") or qk_dim)
         # the one head size the kernels run at
         self.head_dim = qk_dim if v_dim == qk_dim else -(-max(qk_dim, v_dim) // 16) * 16
+        self.v_dim = v_dim
         self.scale = float(params["scale"])
         self.window: Optional[int] = params.get("window")
         if self.num_heads % self.num_kv_heads:
@@ -101,9 +126,36 @@ class PagedAttention(Mixer):
         if self.position.rot_dim > qk_dim:
             raise ValueError("attention: the rotated width exceeds the head size")
 
+        D, nh, nkv = self.head_dim, self.num_heads, self.num_kv_heads
+        self.taps = int(params.get("conv") or 0)
+        self.conv_w = None
+        if self.taps:
+            if not 1 <= self.taps <= 16:
+                raise ValueError(f"attention: {self.taps} taps (1 to 16)")
+            # the taps of every channel of the one product, padded channels with zero taps
+            pads = ((names["q"], nh, qk_dim), (names["k"], nkv, qk_dim), (names["v"], nkv, v_dim))
+            self.conv_w = torch.cat([
+                self._pad_heads(ctx.take(n + ".conv").to(torch.float32), heads, size, D, rows=True)
+                for n, heads, size in pads], dim=0).contiguous()
+        self.head_scales = None
+        if params.get("head_scales"):
+            self.head_scales = ctx.take(join(prefix, params["head_scales"])).to(
+                torch.float32).contiguous()
+        self.softcap = float(params.get("softcap") or 0.0)
+        if self.softcap < 0:
+            raise ValueError(f"attention: softcap {self.softcap} must be positive")
+        mix = params.get("value_mix")
+        self.mix_key = self.mix_source = None
+        self.mix_weight = 0.0
+        if mix:
+            self.mix_key, self.mix_source = str(mix["key"]), bool(mix["source"])
+            # (one number, read once while the model is built)
+            self.mix_weight = float(ctx.take(join(prefix, mix["name"])).to(torch.float32).item())
+
         self.planner = ops.attention_planner(
             self.num_heads, self.num_kv_heads, self.head_dim, self.act_dtype,
-            biased=getattr(self.position, "bias_slopes", None) is not None)
+            biased=getattr(self.position, "bias_slopes", None) is not None,
+            shaped=self.head_scales is not None or self.softcap > 0)
 
     def cache_request(self) -> CacheRequest:
         return CacheRequest.kv(self.num_kv_heads, self.head_dim, self.window)
@@ -111,9 +163,62 @@ class PagedAttention(Mixer):
     def step_planner(self):
         return self.planner
 
+    def state_bytes(self) -> int:
+        """The last ``taps - 1`` rows of the q, k, v product, float32."""
+        if self.taps <= 1:
+            return 0
+        return 4 * (self.taps - 1) * self.w_qkv.shape[0]
+
+    def _project(self, x: Any, step: Any, binding: CacheBinding) -> torch.Tensor:
+        """q, k and v of the step's tokens ``(T, (nh + 2 nkv) D)`` in the activation dtype:
+        the product, and behind it the convolution and the mix of the values where the layer
+        has them."""
+        if not self.taps:
+            qkv = project(x, self.w_qkv, self.act_dtype)
+        else:
+            C = self.w_qkv.shape[0]
+            if isinstance(x, NormedInput) and not ops.can_fuse_norm_linear(
+                    x.stream.x, self.w_qkv, x.stream.x.shape[0]):
+                x = x.tensor()
+            p = (project(x, self.w_qkv, torch.float32) if isinstance(x, NormedInput)
+                 else ops.linear_f32(x, self.w_qkv))
+            if self.taps > 1 and binding.state is None:
+                raise ValueError("attention with a convolution needs a state slot per request; "
+                                 "the runner has none")
+            tail = binding.state.view(torch.float32) if self.taps > 1 else p.new_zeros((1, 1))
+            cu, slots, n = step.cu_seqlens, step.state_slots, step.num_seqs
+            blend = None
+            if self.mix_key is not None and not self.mix_source:
+                handed = step.carried.get(self.mix_key)
+                if handed is None:
+                    raise ValueError(f"attention: no earlier layer of the step handed on values "
+                                     f"under '{self.mix_key}'")
+                blend, heads, size, padded = handed
+                if (heads, size) != (self.num_kv_heads, self.v_dim):
+                    raise ValueError(f"attention: values of {heads} heads of {size} cannot be "
+                                     f"mixed into {self.num_kv_heads} heads of {self.v_dim}")
+                if padded != self.head_dim:      # the two layers pad their heads differently
+                    wide = blend.new_zeros((blend.shape[0], heads, self.head_dim))
+                    wide[:, :, :size] = blend.reshape(-1, heads, padded)[:, :, :size]
+                    blend = wide.reshape(blend.shape[0], heads * self.head_dim)
+            v_from = (self.num_heads + self.num_kv_heads) * self.head_dim
+            qkv = ops.causal_conv(p, self.conv_w, tail, step.seq_of_token, cu, slots, n,
+                                  out_dtype=self.act_dtype, activation=False, blend=blend,
+                                  blend_from=v_from, blend_weight=self.mix_weight)
+            if self.taps > 1:
+                ops.tail_update(tail, p, C, self.taps - 1, cu, slots, n)
+            if self.mix_source:
+                step.carried[self.mix_key] = (qkv[:, v_from:], self.num_kv_heads, self.v_dim,
+                                              self.head_dim)
+            return qkv
+        if self.mix_key is not None:
+            raise ValueError("attention: mixing values across layers is built behind the "
+                             "convolution only")
+        return qkv
+
     def forward(self, x: Any, step: Any, binding: CacheBinding) -> torch.Tensor:
         group = step.groups[binding.group]
-        qkv = project(x, self.w_qkv, self.act_dtype)
+        qkv = self._project(x, step, binding)
         if step.max_context > self.position.max_positions:
             raise ValueError(f"sequence of {step.max_context} positions exceeds max_seq_len "
                              f"{self.position.max_positions}")
@@ -124,5 +229,6 @@ class PagedAttention(Mixer):
                                  write_kv=binding.writes, plan=step.plans.get(self.planner.key()),
                                  interleaved=bool(getattr(self.position, "interleaved", False)),
                                  bias_slopes=getattr(self.position, "bias_slopes", None),
-                                 counters=binding.counters)
+                                 counters=binding.counters, head_scales=self.head_scales,
+                                 softcap=self.softcap)
         return ops.pending_linear(out, self.w_o, self.act_dtype)

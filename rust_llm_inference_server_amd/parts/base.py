@@ -343,8 +343,13 @@ class Block(Part):
 
 
 class Embedding(Part):
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        """Token ids ``(T)`` int32 -> residual stream ``(T, H)`` float32."""
+    # positions the part can place (a table of learned position vectors has so many rows);
+    # None: any
+    position_rows: Optional[int] = None
+
+    def forward(self, ids: torch.Tensor, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Token ids ``(T)`` int32 (and their absolute positions ``(T)`` int32, for a part that
+        adds something per position) -> residual stream ``(T, H)`` float32."""
         raise NotImplementedError
 
 
@@ -374,7 +379,7 @@ class ResidualStream:
     (``round_parts``), as a delta that arrives whole in bfloat16 was by its kernel, so that the
     rounding does not depend on which kernel a batch's size chose."""
 
-    __slots__ = ("x", "pending", "pending_scale", "round_parts")
+    __slots__ = ("x", "pending", "pending_scale", "round_parts", "history")
 
     def __init__(self, x: torch.Tensor, act_dtype: torch.dtype = torch.float32):
         assert x.dtype == torch.float32
@@ -386,6 +391,9 @@ class ResidualStream:
         # adds it); a norm's fused forms take deltas with multiplier 1 only
         self.pending_scale = 1.0
         self.round_parts = act_dtype == torch.bfloat16
+        # (slots, T, H) float32: the embedding output and the layers' results so far, for
+        # blocks that feed the next layer a mix of them (made by the first such block)
+        self.history: Optional[torch.Tensor] = None
 
     def add(self, delta: Any, scale: float = 1.0) -> None:
         if self.pending is not None:

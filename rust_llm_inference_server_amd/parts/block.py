@@ -1,7 +1,10 @@
 """Decoder blocks.  The pre-norm block: ``x += mixer(norm(x)); x += feed_forward(norm(x))``
 (crates/model/src/llama.rs:264-271).  Which mixer, feed-forward and norms it holds, and under
 which weight names, is given by its parameters, layer by layer.  The parallel block:
-``x += mixer(h) + feed_forward(h)`` with ``h = norm(x)``, one norm that both sublayers read."""
+``x += mixer(h) + feed_forward(h)`` with ``h = norm(x)``, one norm that both sublayers read, or
+``x += mixer(norm(x)) + feed_forward(ffn_norm(x))`` with a norm each of the same x.  Behind
+either, optionally, the depth mix: the next layer reads a learned weighted sum of the embedding
+output and of every layer's result so far."""
 from __future__ import annotations
 
 from typing import Any, Dict, List
@@ -68,18 +71,21 @@ class ParallelBlock(Block):
     norm itself (``forward(h, step, resid=..., norm=...)``), for decisions that it wants to make
     on the unrounded input."""
 
-    _SLOTS = (("norm", "norm"), ("mixer", "mixer"), ("feed_forward", "feed_forward"))
+    _SLOTS = (("norm", "norm"), ("mixer", "mixer"), ("feed_forward", "feed_forward"),
+              ("ffn_norm", "norm"))
 
     @classmethod
     def _slots(cls, params: Dict[str, Any]):
-        return cls._SLOTS[:2] if params.get("feed_forward") is None else cls._SLOTS
+        if params.get("feed_forward") is None:
+            return cls._SLOTS[:2]
+        return cls._SLOTS if params.get("ffn_norm") is not None else cls._SLOTS[:3]
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         out: List[TensorSpec] = []
         for slot, category in cls._slots(params):
             out += tensor_specs(category, params[slot], join(prefix, params["names"][slot]))
-        return out
+        return out + DepthMix.tensor_specs(params.get("depth_mix"), prefix)
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
@@ -87,22 +93,71 @@ class ParallelBlock(Block):
                  for slot, category in self._slots(params)}
         self.norm, self.mixer = built["norm"], built["mixer"]
         self.feed_forward = built.get("feed_forward")
+        self.ffn_norm = built.get("ffn_norm")
+        self.depth_mix = DepthMix(params["depth_mix"], prefix, ctx) \
+            if params.get("depth_mix") else None
 
     @property
     def graph_safe(self) -> bool:
-        return all(p.graph_safe for p in (self.norm, self.mixer, self.feed_forward)
-                   if p is not None)
+        return all(p.graph_safe for p in (self.norm, self.mixer, self.feed_forward,
+                                          self.ffn_norm) if p is not None)
 
     def forward(self, stream: ResidualStream, step: Any, binding: CacheBinding) -> None:
         h = self.norm.forward(stream)
         mixed = self.mixer.forward(h, step, binding)
         if self.feed_forward is None:
-            stream.add(mixed)
-            return
-        if getattr(self.feed_forward, "wants_residual", False):
-            # (the norm has folded the pending delta in: stream.x is what it normalised)
-            fed = self.feed_forward.forward(h, step, resid=stream.x, norm=self.norm)
+            delta = mixed
         else:
-            fed = self.feed_forward.forward(h, step)
-        mixed, fed = (d if isinstance(d, torch.Tensor) else d.run() for d in (mixed, fed))
-        stream.add(ops.weighted_sum(mixed, 1.0, fed, 1.0, round_parts=stream.round_parts))
+            # (the first norm has folded the pending delta in: stream.x is what both normalise)
+            h2 = h if self.ffn_norm is None else self.ffn_norm.forward(stream)
+            if getattr(self.feed_forward, "wants_residual", False):
+                fed = self.feed_forward.forward(h2, step, resid=stream.x,
+                                                norm=self.ffn_norm or self.norm)
+            else:
+                fed = self.feed_forward.forward(h2, step)
+            mixed, fed = (d if isinstance(d, torch.Tensor) else d.run() for d in (mixed, fed))
+            delta = ops.weighted_sum(mixed, 1.0, fed, 1.0, round_parts=stream.round_parts)
+        if self.depth_mix is None:
+            stream.add(delta)
+        else:
+            self.depth_mix.apply(stream, delta)
+
+
+class DepthMix:
+    """What a block that names ``depth_mix`` does behind its sublayers: the block's result
+    ``y = x + delta`` is kept beside the embedding output and the results of the layers before
+    it, and the stream becomes ``sum_j w[j] * source_j`` over all of them (source 0 the embedding
+    output, source j the result of the j-th such layer), in float32.
+
+    Parameters: ``weight_name`` (the weights' tensor under the block's prefix, one per source:
+    ``sources`` of them, the number of layers so far plus one) and ``slots`` (sources the model
+    has in all: its layers plus one).  The first such layer (``sources`` 2) makes the history
+    for the step and stores its input as source 0."""
+
+    @staticmethod
+    def tensor_specs(params: Any, prefix: str) -> List[TensorSpec]:
+        if not params:
+            return []
+        return [TensorSpec(join(prefix, params["weight_name"]), (int(params["sources"]),),
+                           init="ones_normal", std=0.3)]
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        self.sources, self.slots = int(params["sources"]), int(params["slots"])
+        if not 2 <= self.sources <= self.slots:
+            raise ValueError(f"depth mix: {self.sources} sources of {self.slots}")
+        self.weights = ctx.take(join(prefix, params["weight_name"])).to(torch.float32).contiguous()
+
+    def apply(self, stream: ResidualStream, delta: Any) -> None:
+        x = stream.flush()
+        if not isinstance(delta, torch.Tensor):
+            delta = delta.run()
+        if delta.dim() == 3 or delta.dtype != torch.float32:
+            delta = ops.weighted_sum(delta, 1.0, None, round_parts=stream.round_parts)
+        first = self.sources == 2
+        if first:
+            stream.history = torch.empty((self.slots, *x.shape), dtype=torch.float32,
+                                         device=x.device)
+        elif stream.history is None:
+            raise ValueError("depth mix: a layer mixes earlier results, but no layer before it "
+                             "kept any")
+        ops.depth_mix_(x, delta, stream.history, self.sources, self.weights, save_input=first)

@@ -17,24 +17,43 @@ from .base import BuildContext, Embedding, Head, TensorSpec, join, project, regi
 @register("embedding", "token")
 class TokenEmbedding(Embedding):
     """Parameters: ``vocab_size``, ``hidden_size``; optional ``scale`` (the rows are multiplied
-    by it as they enter the float32 stream) and ``weight_name`` (the table's name under the
-    prefix, "weight" by default; "" when it is stored under the prefix itself)."""
+    by it as they enter the float32 stream), ``weight_name`` (the table's name under the
+    prefix, "weight" by default; "" when it is stored under the prefix itself) and
+    ``learned_positions``: ``{"name": full tensor name, "rows": positions}``, a table of
+    learned position vectors of which row p is added, unscaled, to the token at position p."""
 
     graph_safe = True
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(join(prefix, params.get("weight_name", "weight")),
-                           (params["vocab_size"], params["hidden_size"]))]
+        out = [TensorSpec(join(prefix, params.get("weight_name", "weight")),
+                          (params["vocab_size"], params["hidden_size"]))]
+        learned = params.get("learned_positions")
+        if learned:
+            out.append(TensorSpec(learned["name"], (learned["rows"], params["hidden_size"])))
+        return out
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         self.weight = ctx.take(join(prefix, params.get("weight_name", "weight")))
         self.vocab_size = int(params["vocab_size"])
         self.scale = float(params.get("scale", 1.0))
+        self.learned = None
+        self.position_rows = None          # positions the part can place (None: any)
+        learned = params.get("learned_positions")
+        if learned:
+            self.learned = ctx.take(learned["name"])
+            if self.learned.dtype != self.weight.dtype:
+                self.learned = self.learned.to(torch.float32).contiguous()
+                self.weight = self.weight.to(torch.float32).contiguous()
+            self.position_rows = int(self.learned.shape[0])
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return ops.embed(ids, self.weight, self.scale)
+    def forward(self, ids: torch.Tensor, positions: Any = None) -> torch.Tensor:
+        if self.learned is None:
+            return ops.embed(ids, self.weight, self.scale)
+        if positions is None:
+            raise ValueError("embedding: learned position vectors need the tokens' positions")
+        return ops.embed(ids, self.weight, self.scale, self.learned, positions)
 
 
 @register("head", "linear")

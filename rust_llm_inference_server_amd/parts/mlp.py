@@ -42,6 +42,47 @@ class SwiGLU(FeedForward):
         return ops.pending_linear(hidden, self.w_down, self.act_dtype)
 
 
+@register("feed_forward", "mlp")
+class DenseMLP(FeedForward):
+    """Two bias-free projections around an activation: ``down(act(up(x)))``.
+
+    Parameters: ``hidden_size``, ``intermediate_size``, ``activation`` ("gelu_tanh": 0.5 z (1 +
+    tanh(sqrt(2 / pi) (z + 0.044715 z^3))), float32 arithmetic on the stored product),
+    ``names`` (the tensors of up and down under the prefix; default ``up_proj.weight`` and
+    ``down_proj.weight``)."""
+
+    graph_safe = True
+    takes_normed_input = True        # the norm in front goes into the up product where it can
+
+    ACTIVATIONS = {"gelu_tanh": ops.gelu_tanh}
+
+    @classmethod
+    def _names(cls, params: Dict[str, Any], prefix: str) -> Dict[str, str]:
+        names = {"up": "up_proj.weight", "down": "down_proj.weight", **(params.get("names") or {})}
+        return {k: join(prefix, v) for k, v in names.items()}
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        H, I = params["hidden_size"], params["intermediate_size"]
+        n = cls._names(params, prefix)
+        return [TensorSpec(n["up"], (I, H)), TensorSpec(n["down"], (H, I))]
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        n = self._names(params, prefix)
+        self.w_up, self.w_down = ctx.take(n["up"]), ctx.take(n["down"])
+        kind = params.get("activation", "gelu_tanh")
+        if kind not in self.ACTIVATIONS:
+            raise ValueError(f"feed-forward 'mlp': activation '{kind}' is not known "
+                             f"(known: {sorted(self.ACTIVATIONS)})")
+        self.activation = self.ACTIVATIONS[kind]
+        self.act_dtype = ctx.act_dtype
+
+    def forward(self, x: Any, step: Any) -> torch.Tensor:
+        hidden = self.activation(project(x, self.w_up, self.act_dtype))
+        return ops.pending_linear(hidden, self.w_down, self.act_dtype)
+
+
 @register("feed_forward", "clamped_glu")
 class ClampedGLU(FeedForward):
     """A gated unit whose branches are bounded before they meet:
@@ -101,7 +142,12 @@ class RoutedSwiGLU(FeedForward):
     ``top``, ``groups`` and ``keep`` (experts stand in ``groups`` equal groups of neighbours;
     only those of the ``keep`` groups with the largest sum of their two best choice scores
     can be chosen), ``scale`` (multiplies the chosen experts' scores, which are not
-    renormalised), ``shared_size`` (None: no shared unit).
+    renormalised), ``shared_size`` (None: no shared unit).  Optional: ``scores`` ("sigmoid",
+    or "softmax" over all experts), ``group_score`` ("top2", or "max": a group's largest
+    score), ``renormalise`` (the chosen experts' weights are divided by their sum + 1e-20),
+    ``correction`` (False: the router has no correction tensor), ``limit`` and ``alpha`` (with a
+    limit the units are of the bounded kind, ``g sigmoid(alpha g) (u + 1)`` with
+    ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``).
 
     Tensors under the prefix: ``router`` (experts, W), ``correction`` (experts: added to the
     sigmoid scores for the choice only), ``e<i>.gate|up`` (F, W), ``e<i>.down`` (W, F),
@@ -122,8 +168,9 @@ class RoutedSwiGLU(FeedForward):
             out += [TensorSpec(join(prefix, f"e{e}.gate"), (F, W)),
                     TensorSpec(join(prefix, f"e{e}.up"), (F, W)),
                     TensorSpec(join(prefix, f"e{e}.down"), (W, F))]
-        out += [TensorSpec(join(prefix, "router"), (E, W), std=0.5),
-                TensorSpec(join(prefix, "correction"), (E,), std=0.1)]
+        out += [TensorSpec(join(prefix, "router"), (E, W), std=0.5)]
+        if params.get("correction", True):
+            out += [TensorSpec(join(prefix, "correction"), (E,), std=0.1)]
         S = params.get("shared_size")
         if S:
             out += [TensorSpec(join(prefix, "shared.gate"), (S, W)),
@@ -135,7 +182,17 @@ class RoutedSwiGLU(FeedForward):
         super().__init__(params, prefix, ctx)
         E = self.experts = int(params["experts"])
         self.top, self.groups, self.keep = int(params["top"]), int(params["groups"]), int(params["keep"])
-        self.scale = float(params["scale"])
+        self.scale = float(params.get("scale", 1.0))
+        self.scores = params.get("scores", "sigmoid")
+        self.group_score = params.get("group_score", "top2")
+        self.renormalise = bool(params.get("renormalise", False))
+        self.limit = float(params.get("limit") or 0.0)
+        self.alpha = float(params.get("alpha", 1.0))
+        if self.scores not in ("sigmoid", "softmax") or self.group_score not in ("top2", "max"):
+            raise ValueError(f"routed_swiglu: unknown scores '{self.scores}' or group score "
+                             f"'{self.group_score}'")
+        if self.limit < 0:
+            raise ValueError(f"routed_swiglu: limit {self.limit} must be positive")
         if E % self.groups or not 1 <= self.keep <= self.groups \
                 or not 1 <= self.top <= self.keep * (E // self.groups):
             raise ValueError(f"routed_swiglu: {E} experts in {self.groups} groups, {self.keep} "
@@ -148,7 +205,9 @@ class RoutedSwiGLU(FeedForward):
                                       for e in range(E)]).contiguous()
         self.w_down = torch.stack([to(pop(f"e{e}.down")) for e in range(E)]).contiguous()
         self.w_router = ctx.take(join(prefix, "router"))
-        self.correction = ctx.take(join(prefix, "correction")).to(torch.float32).contiguous()
+        self.correction = None
+        if params.get("correction", True):
+            self.correction = ctx.take(join(prefix, "correction")).to(torch.float32).contiguous()
         self.w_shared_gate_up = self.w_shared_down = None
         if params.get("shared_size"):
             gate, up = pop("shared.gate"), pop("shared.up")
@@ -166,9 +225,11 @@ class RoutedSwiGLU(FeedForward):
         else:
             logits = ops.linear(x, self.w_router, torch.float32)
         chosen, weights = ops.route(logits, self.correction, self.groups, self.keep, self.top,
-                                    self.scale)
+                                    self.scale, scores=self.scores, group_score=self.group_score,
+                                    renormalise=self.renormalise)
         shared = None
         if self.w_shared_gate_up is not None:
             shared = ops.linear(ops.linear_swiglu(x, self.w_shared_gate_up), self.w_shared_down,
                                 self.act_dtype)
-        return ops.routed_units(x, self.w_gate_up, self.w_down, chosen, weights, shared)
+        return ops.routed_units(x, self.w_gate_up, self.w_down, chosen, weights, shared,
+                                limit=self.limit, alpha=self.alpha)

@@ -22,7 +22,8 @@ class RMSNorm(Norm):
     """Parameters: ``size`` (hidden width), ``eps``; optional ``weight_offset`` (a number added
     to the stored weight, in float32, once at build time: 1 for weights stored around zero) and
     ``weight_name`` (the tensor's name under the prefix, "weight" by default; "" when the
-    tensor is stored under the prefix itself)."""
+    tensor is stored under the prefix itself); ``scalar``: the stored weight is one number that
+    multiplies every coordinate (a tensor without axes)."""
 
     graph_safe = True
 
@@ -33,12 +34,17 @@ class RMSNorm(Norm):
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         init = "normal" if float(params.get("weight_offset", 0.0)) else "ones_normal"
-        return [TensorSpec(cls._weight_name(params, prefix), (params["size"],), init=init)]
+        shape = () if params.get("scalar") else (params["size"],)
+        return [TensorSpec(cls._weight_name(params, prefix), shape, init=init)]
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         self.eps = float(params["eps"])
         self.weight = ctx.take(self._weight_name(params, prefix))
+        if params.get("scalar"):
+            # the kernels take one weight per coordinate: the one number, float32, repeated
+            self.weight = self.weight.to(torch.float32).reshape(1).expand(
+                int(params["size"])).contiguous()
         offset = float(params.get("weight_offset", 0.0))
         if offset:
             self.weight = (self.weight.to(torch.float32) + offset).contiguous()

@@ -20,6 +20,10 @@ that feed it store float32 results.
 numbers per channel decays by ``exp(dt A)`` with a step ``dt`` that the token chooses, takes
 ``dt x B`` and is read with ``C``; the result is gated by ``silu(z)``.
 
+``decay_attention`` (linear attention with a fixed decay per head): q, k and v pass SiLU; per
+head ``S <- decay_h S + k v^T`` and the read-out ``S^T q`` includes the token's own key and
+value; the heads' read-outs are normalised together, gated by a sigmoid and projected.
+
 ``parallel``: two mixers read the same input, and their outputs meet as a weighted sum in
 float32.  Each keeps what it keeps: the pages of the one that asks for a cache, the state
 bytes of both, one after the other.
@@ -269,6 +273,94 @@ class SelectiveScan(Mixer):
         y = ops.selective_scan(xc, dt_raw, self.dt_bias, low[:, rank:rank + N],
                                low[:, rank + N:rank + 2 * N], xz[:, C:], self.a_log, self.skip,
                                S, cu, slots, n)
+        return ops.pending_linear(y, self.w_o, self.act_dtype)
+
+
+# ----------------------------------------------------------------------- decay attention
+@register("mixer", "decay_attention")
+class DecayAttention(Mixer):
+    """Parameters: ``hidden_size``, ``num_heads``, ``head_dim`` (queries and keys),
+    ``value_dim``, ``decay`` (one number in (0, 1] per head), ``eps`` (of the norm over the
+    concatenated heads).
+
+    Tensors under the prefix: ``q``, ``k`` (heads * d, W), ``v``, ``g`` (heads * dv, W),
+    ``norm`` (heads * dv), ``o`` (W, heads * dv).
+
+    Per token: ``q, k, v = silu(W h)``; per head ``S <- decay_h S + k v^T``, ``o = S^T q`` (no
+    other scale); the concatenated heads are divided by their root mean square, multiplied by
+    ``norm`` and by ``sigmoid(W_g h)``, and projected by ``o``.  One product makes q, k, v and
+    the gate (rows concatenated), stored in float32; SiLU, the state (float32, in the request's
+    slot, [head][value channel][key channel]), the norm and the gate are float32 in either
+    activation dtype."""
+
+    graph_safe = True
+    takes_normed_input = True        # the norm in front goes into the one input product where it can
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        W, H = params["hidden_size"], params["num_heads"]
+        d, dv = params["head_dim"], params["value_dim"]
+        return [TensorSpec(join(prefix, "q"), (H * d, W)), TensorSpec(join(prefix, "k"), (H * d, W)),
+                TensorSpec(join(prefix, "v"), (H * dv, W)), TensorSpec(join(prefix, "g"), (H * dv, W)),
+                TensorSpec(join(prefix, "o"), (W, H * dv)),
+                TensorSpec(join(prefix, "norm"), (H * dv,), init="ones_normal")]
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        self.width = int(params["hidden_size"])
+        self.heads = int(params["num_heads"])
+        self.dim, self.vdim = int(params["head_dim"]), int(params["value_dim"])
+        self.eps = float(params["eps"])
+        decay = [float(x) for x in params["decay"]]
+        if len(decay) != self.heads or not all(0.0 < x <= 1.0 for x in decay):
+            raise ValueError(f"decay_attention: {self.heads} heads need a decay in (0, 1] each, "
+                             f"got {decay}")
+        if self.dim > 256:
+            raise ValueError(f"decay_attention: heads of {self.dim} key channels (at most 256)")
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=ctx.device)
+        take = lambda n: ctx.weights.pop(join(prefix, n))
+        parts = [take("q"), take("k"), take("v"), take("g")]
+        if len({p.dtype for p in parts}) > 1:
+            parts = [p.to(torch.float32) for p in parts]
+        # column ranges of the one product: q | k | v | gate, each from a multiple of 8
+        self.cols: Dict[str, int] = {}
+        rows, at = [], 0
+        for name, p in zip("qkvg", parts):
+            pad = -at % 8
+            if pad:
+                rows.append(p.new_zeros((pad, self.width)))
+                at += pad
+            self.cols[name] = at
+            rows.append(p)
+            at += p.shape[0]
+        if at % 8:
+            rows.append(parts[0].new_zeros((-at % 8, self.width)))
+        self.w_in = torch.cat(rows, dim=0).contiguous()
+        del parts, rows
+        self.norm = _f32(ctx.take(join(prefix, "norm")))
+        self.w_o = ctx.take(join(prefix, "o"))
+        self.act_dtype = ctx.act_dtype
+
+    def state_bytes(self) -> int:
+        return 4 * self.heads * self.vdim * self.dim
+
+    def forward(self, x: Any, step: Any, binding: CacheBinding) -> Any:
+        H, d, dv = self.heads, self.dim, self.vdim
+        if binding.state is None:
+            raise ValueError("decay_attention needs a state slot per request; the runner has none")
+        S = binding.state.view(torch.float32)
+        cu, slots, n = step.cu_seqlens, step.state_slots, step.num_seqs
+        if isinstance(x, NormedInput) and not ops.can_fuse_norm_linear(
+                x.stream.x, self.w_in, x.stream.x.shape[0]):
+            x = x.tensor()
+        p = (project(x, self.w_in, torch.float32) if isinstance(x, NormedInput)
+             else ops.linear_f32(x, self.w_in))                           # (T, q | k | v | gate)
+        c = self.cols
+        o = ops.decay_attention(p[:, c["q"]:c["q"] + H * d], p[:, c["k"]:c["k"] + H * d],
+                                p[:, c["v"]:c["v"] + H * dv], self.decay, S, cu, slots, n,
+                                H, d, dv)
+        y = ops.head_norm_gate(o, self.norm, p[:, c["g"]:c["g"] + H * dv], 1, H * dv, self.eps,
+                               self.act_dtype, sigmoid_gate=True)
         return ops.pending_linear(y, self.w_o, self.act_dtype)
 
 

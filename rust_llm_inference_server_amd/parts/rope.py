@@ -5,7 +5,9 @@ Inverse frequencies are computed in float32 exactly as the reference does
 whose wavelength is below ``original / high_freq_factor`` is kept, one above
 ``original / low_freq_factor`` is divided by ``factor``, and those between are blended.
 Angles ``position * inv_freq``, cosines and sines are float32 (rope.rs:61-78) and stay so:
-the table is never rounded to the activation dtype.  The rotation pairs dim ``j`` with
+the table is never rounded to the activation dtype.  A second kind of scaling, ``yarn``,
+stretches the slow frequencies by ``factor``, keeps the fast ones, blends those between along
+a ramp over the pair index, and multiplies cosines and sines by ``0.1 ln(factor) + 1``.  The rotation pairs dim ``j`` with
 ``j + rot/2`` (rotate-half, rope.rs:111-117) and is applied by the cache-write kernel."""
 from __future__ import annotations
 
@@ -15,6 +17,29 @@ from typing import Any, Dict, Optional
 import torch
 
 from .base import BuildContext, PositionEncoding, register
+
+
+def yarn_frequencies(rot_dim: int, theta: float, scaling: Dict[str, Any]) -> torch.Tensor:
+    """Frequencies of pair i = 0 .. rot_dim / 2 - 1 in double precision.  With ``turns(n)`` the
+    (fractional) pair index whose wave makes n turns over ``original`` positions,
+    ``rot_dim ln(original / (2 pi n)) / (2 ln theta)``: pairs up to ``lo = floor(turns(fast))``
+    keep ``f_i = theta^(-2 i / rot_dim)``, pairs from ``hi = ceil(turns(slow))`` on get
+    ``f_i / factor``, and between the two the share of the stretched frequency rises linearly."""
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+    fast, slow = float(scaling["fast"]), float(scaling["slow"])
+    if not (factor > 0 and original > 0 and fast > 0 and slow > 0):
+        raise ValueError("position encoding 'rope': yarn scaling needs positive 'factor', "
+                         "'original', 'fast' and 'slow'")
+
+    def turns(n: float) -> float:
+        return rot_dim * math.log(original / (2.0 * math.pi * n)) / (2.0 * math.log(theta))
+
+    lo = max(math.floor(turns(fast)), 0)
+    hi = min(math.ceil(turns(slow)), rot_dim - 1)
+    i = torch.arange(0, rot_dim // 2, dtype=torch.float64)
+    f = float(theta) ** (-2.0 * i / rot_dim)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return f / factor * ramp + f * (1.0 - ramp)
 
 
 def inverse_frequencies(rot_dim: int, theta: float, scaling: Optional[Dict[str, Any]]
@@ -42,19 +67,26 @@ def inverse_frequencies(rot_dim: int, theta: float, scaling: Optional[Dict[str, 
 @register("position", "rope")
 class RotaryEmbedding(PositionEncoding):
     """Parameters: ``rot_dim`` (rotated width, at most the head size), ``theta``, ``scaling``
-    (None or the llama3 fields).  Holds ``cos``/``sin`` float32 ``(max_positions, rot/2)``.
+    (None, the llama3 fields, or ``{"rope_type": "yarn", "factor", "original", "fast",
+    "slow"}``).  Holds ``cos``/``sin`` float32 ``(max_positions, rot/2)``.
     Optional ``precise``: frequencies, angles, cosines and sines are made in double precision
     and rounded once to float32 (without it they are float32 from the start, as the reference
-    makes them)."""
+    makes them); yarn scaling is always made that way."""
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         rot = int(params["rot_dim"])
         if rot % 2:
             raise ValueError(f"position encoding 'rope': rot_dim {rot} must be even")
-        if params.get("precise"):
-            if params.get("scaling"):
-                raise ValueError("position encoding 'rope': 'precise' has no frequency scaling")
+        scaling = params.get("scaling")
+        magnitude = 1.0
+        if scaling and scaling.get("rope_type") == "yarn":
+            inv = yarn_frequencies(rot, float(params["theta"]), scaling)
+            magnitude = 0.1 * math.log(float(scaling["factor"])) + 1.0
+            pos = torch.arange(ctx.max_positions, dtype=torch.float64).reshape(-1, 1)
+        elif params.get("precise"):
+            if scaling:
+                raise ValueError("position encoding 'rope': 'precise' has no llama3 scaling")
             f64 = torch.float64
             inv = float(params["theta"]) ** (-torch.arange(0, rot, 2, dtype=f64) / rot)
             pos = torch.arange(ctx.max_positions, dtype=f64).reshape(-1, 1)
@@ -64,8 +96,8 @@ class RotaryEmbedding(PositionEncoding):
         angles = pos * inv.reshape(1, -1)
         self.rot_dim = rot
         self.inv_freq = inv.to(torch.float32)
-        self.cos = torch.cos(angles).to(torch.float32).to(ctx.device).contiguous()
-        self.sin = torch.sin(angles).to(torch.float32).to(ctx.device).contiguous()
+        self.cos = (torch.cos(angles) * magnitude).to(torch.float32).to(ctx.device).contiguous()
+        self.sin = (torch.sin(angles) * magnitude).to(torch.float32).to(ctx.device).contiguous()
         self.max_positions = ctx.max_positions
 
 
