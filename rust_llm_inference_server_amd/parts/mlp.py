@@ -54,7 +54,7 @@ class DenseMLP(FeedForward):
     graph_safe = True
     takes_normed_input = True        # the norm in front goes into the up product where it can
 
-    ACTIVATIONS = {"gelu_tanh": ops.gelu_tanh}
+    ACTIVATIONS = {"gelu_tanh": "gelu_tanh"}       # activation -> the kernel's name in ops
 
     @classmethod
     def _names(cls, params: Dict[str, Any], prefix: str) -> Dict[str, str]:
@@ -79,7 +79,7 @@ class DenseMLP(FeedForward):
         self.act_dtype = ctx.act_dtype
 
     def forward(self, x: Any, step: Any) -> torch.Tensor:
-        hidden = self.activation(project(x, self.w_up, self.act_dtype))
+        hidden = getattr(ops, self.activation)(project(x, self.w_up, self.act_dtype))
         return ops.pending_linear(hidden, self.w_down, self.act_dtype)
 
 

@@ -12,8 +12,37 @@ from __future__ import annotations
 import torch
 
 
-def embed(ids, table, scale=1.0):
-    return table[ids.long()].to(torch.float32) * scale
+def embed(ids, table, scale=1.0, learned=None, positions=None):
+    out = table[ids.long()].to(torch.float32) * scale
+    return out if learned is None else out + learned[positions.long()].to(torch.float32)
+
+
+def gelu_tanh(x):
+    z = x.float()
+    return (0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))).to(x.dtype)
+
+
+def depth_mix_(x, delta, history, count, weights, save_input=False):
+    if save_input:
+        history[0] = x
+    history[count - 1] = x + delta
+    x.copy_(sum(weights[j].float() * history[j] for j in range(count)))
+
+
+def decay_attention(q, k, v, decay, state, cu, slots, num_seqs, heads, dim, vdim, activation=True):
+    T = q.shape[0]
+    act = (lambda z: z / (1.0 + torch.exp(-z))) if activation else (lambda z: z)
+    qq, kk = act(q.float()).reshape(T, heads, dim), act(k.float()).reshape(T, heads, dim)
+    vv = act(v.float()).reshape(T, heads, vdim)
+    out = torch.empty((T, heads * vdim), dtype=torch.float32)
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        S = state[slot, :heads * vdim * dim].reshape(heads, vdim, dim).clone()   # [head][value][key]
+        for t in range(t0, t1):
+            for h in range(heads):
+                S[h] = decay[h] * S[h] + torch.outer(vv[t, h], kk[t, h])
+                out[t, h * vdim:(h + 1) * vdim] = S[h] @ qq[t, h]
+        state[slot, :heads * vdim * dim] = S.reshape(-1)
+    return out
 
 
 def add_residual(resid, delta, round_parts=False, delta_scale=1.0):
@@ -88,7 +117,8 @@ def tail_update(state, x, channels, rows, cu, slots, num_seqs):
 
 def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels=0, unit_group=0,
                 scaled_channels=0, scale=1.0, unit_eps=0.0, rest_group=256, bias=None,
-                out_dtype=torch.float32):
+                out_dtype=torch.float32, activation=True, blend=None, blend_from=0,
+                blend_weight=0.0):
     C, K = taps.shape
     out = torch.empty((x.shape[0], C), dtype=torch.float32)
     for t0, t1, slot in _seqs(cu, slots, num_seqs):
@@ -96,7 +126,9 @@ def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels
         acc = torch.zeros(t1 - t0, C) if bias is None else bias.reshape(1, C).repeat(t1 - t0, 1)
         for j in range(K):
             acc += both[j:j + t1 - t0] * taps[:, j]
-        out[t0:t1] = acc / (1.0 + torch.exp(-acc))
+        out[t0:t1] = acc / (1.0 + torch.exp(-acc)) if activation else acc
+    if blend is not None:
+        out[:, blend_from:] = (1.0 - blend_weight) * out[:, blend_from:] + blend_weight * blend.float()
     if unit_channels:
         y = out[:, :unit_channels].reshape(x.shape[0], -1, unit_group)
         y = y / torch.sqrt((y * y).sum(-1, keepdim=True) + unit_eps)
@@ -218,26 +250,34 @@ def router_logits(resid, norm_weight, norm_bias, eps, w_router):
     return h @ w_router.float().t()
 
 
-def route(logits, correction, groups, keep, top, scale):
+def route(logits, correction, groups, keep, top, scale, scores="sigmoid", group_score="top2",
+          renormalise=False):
     T, E = logits.shape
-    s = torch.sigmoid(logits)
-    choice = (s + correction).reshape(T, groups, E // groups)
-    score = choice.topk(min(2, E // groups), dim=-1).values.sum(-1)
+    s = torch.sigmoid(logits) if scores == "sigmoid" else torch.softmax(logits, dim=-1)
+    choice = (s if correction is None else s + correction).reshape(T, groups, E // groups)
+    score = choice.topk(1 if group_score == "max" else min(2, E // groups), dim=-1).values.sum(-1)
     kept = torch.zeros(T, groups, dtype=torch.bool)
     kept.scatter_(1, score.topk(keep, dim=-1).indices, True)
     choice = choice.masked_fill(~kept.unsqueeze(-1), float("-inf")).reshape(T, E)
     chosen = choice.topk(top, dim=-1).indices
-    return chosen.to(torch.int32), (s.gather(1, chosen) * scale).float()
+    weights = (s.gather(1, chosen) * scale).float()
+    if renormalise:
+        weights = weights / (weights.sum(-1, keepdim=True) + 1e-20)
+    return chosen.to(torch.int32), weights
 
 
-def routed_units(x, w_gate_up, w_down, chosen, weights, addend=None):
+def routed_units(x, w_gate_up, w_down, chosen, weights, addend=None, limit=0.0, alpha=1.0):
     T, W = x.shape
     F = w_gate_up.shape[1] // 2
     out = torch.zeros(T, W)
     for t in range(T):
         for e, wt in zip(chosen[t].tolist(), weights[t].tolist()):
             gu = w_gate_up[e].float() @ x[t].float()
-            hidden = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(x.dtype).float()
+            if limit > 0:
+                g, u = gu[:F].clamp(max=limit), gu[F:].clamp(-limit, limit)
+                hidden = (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(x.dtype).float()
+            else:
+                hidden = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(x.dtype).float()
             out[t] += wt * (w_down[e].float() @ hidden)
     return out if addend is None else out + addend.float()
 
@@ -279,13 +319,14 @@ def decay_scan(r, k, v, z, w0, bonus, state, cu, slots, num_seqs, heads, d, tile
     return out
 
 
-def head_norm_gate(o, weight, gate, heads, dv, eps, out_dtype):
+def head_norm_gate(o, weight, gate, heads, dv, eps, out_dtype, sigmoid_gate=False):
     T = o.shape[0]
     x = o.reshape(T, heads, dv)
     x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
     w = weight.reshape(heads, dv) if weight.numel() == heads * dv else weight.reshape(1, dv)
     g = gate.float().reshape(T, heads, dv)
-    return (x * w * (g / (1.0 + torch.exp(-g)))).reshape(T, heads * dv).to(out_dtype)
+    g = torch.sigmoid(g) if sigmoid_gate else g / (1.0 + torch.exp(-g))
+    return (x * w * g).reshape(T, heads * dv).to(out_dtype)
 
 
 def linear(x, w, out_dtype=None, partials=False):
@@ -334,14 +375,14 @@ def copy_pages(pages, src, dst):
         pages[:, d] = pages[:, s]
 
 
-def attention_planner(num_heads, num_kv_heads, head_dim, dtype, biased=False):
+def attention_planner(num_heads, num_kv_heads, head_dim, dtype, biased=False, shaped=False):
     from rust_llm_inference_server_amd.ops.attention_plan import AttentionPlanner
     return AttentionPlanner(num_heads, num_kv_heads, head_dim, matrix=dtype == torch.bfloat16)
 
 
 def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
                     block_tables, step, scale, window=None, force=None, plan=None,
-                    bias_slopes=None, counters=None):
+                    bias_slopes=None, counters=None, head_scales=None, softcap=0.0):
     assert bias_slopes is None, "the test double adds no bias"
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
@@ -358,6 +399,10 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
         v = torch.stack([v_pages[table[p // page_size], :, :, p % page_size] for p in keys]).float()
         for h in range(nh):
             s = (k[:, h // g, :] @ q[t, h]) * scale
+            if head_scales is not None:
+                s = s * head_scales[h]
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
             p = torch.softmax(s, dim=0)
             out[t, h * d:(h + 1) * d] = p @ v[:, h // g, :]
     return out.to(qkv.dtype)
@@ -365,11 +410,13 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
 
 def rope_attention(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                    v_pages, page_size, block_tables, step, scale, window=None, write_kv=True,
-                   plan=None, interleaved=False, bias_slopes=None, counters=None):
+                   plan=None, interleaved=False, bias_slopes=None, counters=None,
+                   head_scales=None, softcap=0.0):
     rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                   v_pages, page_size, write_kv=write_kv)
     return paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
-                           block_tables, step, scale, window)
+                           block_tables, step, scale, window, head_scales=head_scales,
+                           softcap=softcap)
 
 
 def _lowbias32(x):
@@ -410,6 +457,7 @@ def install(monkeypatch) -> None:
                  "causal_conv", "delta_scan", "decay_scan", "head_norm_gate", "selective_scan",
                  "add_layernorm", "scale_", "head_linear", "latent_write", "latent_attention",
                  "latent_mfma_ok",
-                 "sigmoid_gate_", "route", "routed_units", "router_logits"):
+                 "sigmoid_gate_", "route", "routed_units", "router_logits", "gelu_tanh",
+                 "depth_mix_", "decay_attention"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))
