@@ -232,6 +232,11 @@ class LagedraConfig:
     def vocab_size(self) -> int:
         return self.vocab
 
+    @property
+    def max_position_embeddings(self) -> int:
+        """The longest sequence the model can place: one learned vector per position."""
+        return self.max_positions
+
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "LagedraConfig":
         where = "config.json"

@@ -41,8 +41,8 @@ class PagedAttention(Mixer):
       step under ``key``; every other layer with that key replaces its values by
       ``(1 - w) v + w v_source`` (``w`` the tensor's one number) before they are cached.
 
-    With ``value_dim != head_dim`` the kernels run at one head size ``D``, the larger of the two
-    rounded up to a multiple of 16: the rows of the narrower projection's weight are padded
+    With ``value_dim != head_dim`` (or an odd head size) the kernels run at one head size ``D``,
+    the larger of the two rounded up to a multiple of 16: the rows of the narrower projection's weight are padded
     with zero rows per head at build time (and the output projection's columns with zero
     columns), so the extra query and key dims add exact zeros to every score and the extra
     value dims come out as exact zeros that meet zero columns.  The kernels stay specialised on
@@ -102,7 +102,9 @@ class PagedAttention(Mixer):
         qk_dim = int(params["head_dim"])
         v_dim = int(params.get("value_dim") or qk_dim)
         # the one head size the kernels run at
-        self.head_dim = qk_dim if v_dim == qk_dim else -(-max(qk_dim, v_dim) // 16) * 16
+        # (equal sizes stay as they are when the kernels take them: even head sizes)
+        self.head_dim = qk_dim if v_dim == qk_dim and qk_dim % 2 == 0 \
+            else -(-max(qk_dim, v_dim) // 16) * 16
         self.v_dim = v_dim
         self.scale = float(params["scale"])
         self.window: Optional[int] = params.get("window")

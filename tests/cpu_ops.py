@@ -122,7 +122,8 @@ def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels
     C, K = taps.shape
     out = torch.empty((x.shape[0], C), dtype=torch.float32)
     for t0, t1, slot in _seqs(cu, slots, num_seqs):
-        both = torch.cat([state[slot, :C * (K - 1)].reshape(K - 1, C), x[t0:t1, :C].float()], dim=0)
+        before = state[slot, :C * (K - 1)].reshape(K - 1, C) if K > 1 else x.new_zeros((0, C))
+        both = torch.cat([before.float(), x[t0:t1, :C].float()], dim=0)
         acc = torch.zeros(t1 - t0, C) if bias is None else bias.reshape(1, C).repeat(t1 - t0, 1)
         for j in range(K):
             acc += both[j:j + t1 - t0] * taps[:, j]
