@@ -91,9 +91,24 @@ __host__ __device__ constexpr int tile_bufs(int QB) {
 
 // Up to three waves per SIMD (two with two query blocks): the staging registers must not be
 // traded for another.
+// A score of the shaped forms in the base-2 domain: the raw product times the head's scale,
+// under a cap c > 0 as c * tanh(score / c) (tanh x = 1 - 2 / (1 + e^(2x)), float32), plus the
+// bias term (already in the base-2 domain).
+__device__ __forceinline__ float shaped_score(float raw, float scale, float cap, float inv_cap,
+                                              float bias2) {
+  float v = raw * scale;
+  if (cap > 0.f) {
+    const float e = __builtin_amdgcn_exp2f(v * inv_cap * 2.8853900817779268f);
+    v = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
+  }
+  return fmaf(v, 1.4426950408889634f, bias2);
+}
+
 // BIAS: a bias on the scores, slopes[head] * (key position - query position) added in float32
-// before the softmax (the reference has none; a position encoding of another kind has).  A form
-// of its own, so that the usual one pays nothing for it.
+// before the softmax (the reference has none; a position encoding of another kind has), and
+// the other shapings of a score: head_scales[head] on top of the scale, and a cap
+// c * tanh(score / c).  Any of the three may be absent (null, 0).  A form of its own, so that
+// the usual one pays nothing for it.
 template <int QB, bool BIAS = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 && D <= 64) ? 4 : 1, QB == 1 ? (D <= 64 ? 4 : 3) : (D <= 64 ? 3 : 2)))) void KERNEL_NAME(
     const bf16_t* __restrict__ q, long long q_stride, bf16_t* __restrict__ out,
@@ -103,7 +118,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int part_stride,
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    const float* __restrict__ slopes) {
+    const float* __restrict__ slopes, const float* __restrict__ head_scales, float softcap) {
   constexpr int BN = tile_keys(QB);
   // V^T tile rows: 64 keys padded to a stride of 32 bytes mod 64; 32 keys unpadded, with the
   // 16-byte piece index XORed with (-(row / 4)) & 3, which frees reads and stores of conflicts.
@@ -292,7 +307,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   const float scale2 = scale * 1.4426950408889634f;      // scores in the base-2 domain
   // With a bias the scores are brought to the base-2 domain as soon as they are formed
   // (score * scale2 + slope2 * distance), and maximum and exponent take them as they are.
-  const float slope2 = BIAS ? slopes[h] * 1.4426950408889634f : 0.f;
+  const float slope2 = (BIAS && slopes) ? slopes[h] * 1.4426950408889634f : 0.f;
+  // (the same form shapes the scores: a number per head on top of the scale, and a cap)
+  const float shaped = (BIAS && head_scales) ? scale * head_scales[h] : scale;
+  const float inv_cap = (BIAS && softcap > 0.f) ? 1.0f / softcap : 0.f;
   const float in_exp = BIAS ? 1.f : scale2;
   if (kt0 < khi) {           // else this run has no keys (only with splits)
   RLIS_LOAD_PAGES(kt0, page_ka, page_va);
@@ -359,7 +377,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const int kpos = k0 + (nb / 2) * 32 + lq * 8 + 2 * r + (nb % 2);
-              s[b][nb][r] = fmaf(s[b][nb][r], scale2, slope2 * (float)(kpos - my_qpos[b]));
+              s[b][nb][r] = shaped_score(s[b][nb][r], shaped, softcap, inv_cap,
+                                         slope2 * (float)(kpos - my_qpos[b]));
             }
       }
       // ---- scale, mask (only where a tile meets the diagonal, the window or the end) -----
@@ -527,8 +546,9 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
     int page_shift, int window, float scale, int tile_queries, int splits, int row0,
     float* part_ml, float* part_acc, const float* cos, const float* sin, int rot,
-    const float* slopes, hipStream_t stream) {
+    const float* slopes, const float* head_scales, float softcap, hipStream_t stream) {
   if (num_tiles == 0) return 0;
+  const bool shaped = slopes || head_scales || softcap > 0.f;
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
   if (cos && !(sin && D % 64 == 0 && rot == D && d == D)) return kUnitBadRotation;
   const long long blocks = (long long)num_tiles * nh;
@@ -540,12 +560,12 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,              \
       (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, \
       d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, \
-      cos, sin, slopes)
+      cos, sin, slopes, head_scales, softcap)
   if (tile_queries == 2 * BM) {
-    if (slopes) RLIS_PREFILL_LAUNCH(2, true);
+    if (shaped) RLIS_PREFILL_LAUNCH(2, true);
     else RLIS_PREFILL_LAUNCH(2, false);
   } else {
-    if (slopes) RLIS_PREFILL_LAUNCH(1, true);
+    if (shaped) RLIS_PREFILL_LAUNCH(1, true);
     else RLIS_PREFILL_LAUNCH(1, false);
   }
 #undef RLIS_PREFILL_LAUNCH
@@ -645,7 +665,8 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
     int max_parts, int merge_inside, int groups, int cap, const DecodeRope rope,
-    const DecodeMerge merge, const float* __restrict__ slopes) {
+    const DecodeMerge merge, const float* __restrict__ slopes,
+    const float* __restrict__ head_scales, float softcap) {
   if constexpr (EXACT) {
     d = D;
     page_shift = kExactPageShift;
@@ -824,7 +845,9 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   for (int db = 0; db < D / 16; ++db) o_acc[db] = (f32x4){0.f, 0.f, 0.f, 0.f};
   const float scale2 = scale * 1.4426950408889634f;
   // (with a bias the scores go to the base-2 domain as they are formed, see the prefill kernel)
-  const float slope2 = BIAS ? slopes[kvh * g + min(l16, g - 1)] * 1.4426950408889634f : 0.f;
+  const float slope2 = (BIAS && slopes) ? slopes[kvh * g + min(l16, g - 1)] * 1.4426950408889634f : 0.f;
+  const float shaped = (BIAS && head_scales) ? scale * head_scales[kvh * g + min(l16, g - 1)] : scale;
+  const float inv_cap = (BIAS && softcap > 0.f) ? 1.0f / softcap : 0.f;
   const float in_exp = BIAS ? 1.f : scale2;
 
   auto compute = [&](int c0, const Frag8 (&kf)[2][D / 32], const Frag8 (&vf)[D / 16])
@@ -843,7 +866,9 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = c0 + nb * 16 + lq * 4 + r;
-        if constexpr (BIAS) s[nb][r] = fmaf(s[nb][r], scale2, slope2 * (float)(key - (ctx - 1)));
+        if constexpr (BIAS)
+          s[nb][r] = shaped_score(s[nb][r], shaped, softcap, inv_cap,
+                                  slope2 * (float)(key - (ctx - 1)));
         const float sv = (key >= lo && key < kend) ? s[nb][r] : -INFINITY;
         s[nb][r] = sv;
         mx = fmaxf(mx, sv);
@@ -1081,8 +1106,10 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     float* part_acc, const void* k_pages, const void* v_pages, const int* block_tables,
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
     float scale, int splits, int part_keys, int max_parts, int merge_inside, int groups, int cap,
-    const DecodeRope* rope, const DecodeMerge* merge, const float* slopes, hipStream_t stream) {
+    const DecodeRope* rope, const DecodeMerge* merge, const float* slopes,
+    const float* head_scales, float softcap, hipStream_t stream) {
   if (S == 0) return 0;
+  const bool shaped = slopes || head_scales || softcap > 0.f;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
   if (merge_inside && (!merge->arrivals || (long long)S * nkv > merge->slots))
     return kUnitTooManyArrivals;
@@ -1124,10 +1151,10 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,                   \
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
       d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, groups, cap,   \
-      *rope, *merge, slopes)
+      *rope, *merge, slopes, head_scales, softcap)
   const bool exact = d == D && page_shift == kExactPageShift && window <= 0;
-  if (slopes && cap > 1) RLIS_DEC_LAUNCH(true, false, true);
-  else if (slopes) RLIS_DEC_LAUNCH(false, false, true);
+  if (shaped && cap > 1) RLIS_DEC_LAUNCH(true, false, true);
+  else if (shaped) RLIS_DEC_LAUNCH(false, false, true);
   else if (cap > 1 && exact) RLIS_DEC_LAUNCH(true, true, false);
   else if (cap > 1) RLIS_DEC_LAUNCH(true, false, false);
   else if (exact) RLIS_DEC_LAUNCH(false, true, false);

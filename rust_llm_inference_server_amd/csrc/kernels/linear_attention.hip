@@ -12,9 +12,11 @@
 //    head), lane i holds S[.][i + 64 r]; the next token's inputs are asked for before the
 //    current token's sums.  Decode steps and short portions.
 //  * decay_attention_chunks: long portions in chunks of 64 tokens on the matrix cores (float32
-//    products): a chunk's own contribution to the state, a sequential pass over the chunks that
-//    leaves every chunk's start state, and the chunk's read-outs
-//    O = (Q K^T . D) V + diag(decay^(t+1)) Q S_start with D[t][s] = decay^(t-s) for s <= t.
+//    products, v_mfma_f32_16x16x4_f32): a chunk's own contribution to the state, a pass over
+//    each sequence's chunks in order that leaves every chunk's start state, and the chunk's
+//    read-outs O = (Q K^T . D) V + diag(decay^(t+1)) Q S_start with D[t][s] = decay^(t-s) for
+//    s <= t.  Chunks and heads run side by side; only the join is sequential, and it is one
+//    multiply-add per state element and chunk.
 #include "common.h"
 #include "tile_mma.h"
 
@@ -104,6 +106,228 @@ __global__ __launch_bounds__(256) void decay_attention_scan_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------- chunked form
+constexpr int kChunk = 64;           // tokens a chunk
+constexpr int kTokStride = kChunk + 4;   // floats between rows that run along the tokens
+
+__device__ __forceinline__ int round16(int n) { return (n + 15) / 16 * 16; }
+
+// The b-th chunk of the step, counting every sequence's chunks of kChunk tokens in order:
+// its sequence, its number inside it, its first token and how many it holds.  False: the step
+// has fewer chunks.
+struct ChunkAt {
+  int seq, index, first, count, chunks_before_seq;
+};
+
+__device__ __forceinline__ bool find_chunk(const int* __restrict__ cu, int S, int b, ChunkAt& at) {
+  int seen = 0;
+  for (int s = 0; s < S; ++s) {
+    const int t0 = cu[s], len = cu[s + 1] - t0;
+    const int nc = (len + kChunk - 1) / kChunk;
+    if (b < seen + nc) {
+      at.seq = s;
+      at.index = b - seen;
+      at.first = t0 + at.index * kChunk;
+      at.count = min(kChunk, t0 + len - at.first);
+      at.chunks_before_seq = seen;
+      return true;
+    }
+    seen += nc;
+  }
+  return false;
+}
+
+// What a chunk of n tokens adds to the state, from a zero state: A[j][i] = sum_s decay^(n-1-s)
+// k_s[i] v_s[j], the product over the tokens of V^T and of K^T with the decays folded in, both
+// transposed into LDS.  grid (chunks, heads); ws holds (chunk, head, value channel, key
+// channel).
+__global__ __launch_bounds__(256) void decay_chunk_states_kernel(
+    float* __restrict__ ws, const float* __restrict__ k, long long ldk,
+    const float* __restrict__ v, long long ldv, const float* __restrict__ decay,
+    const int* __restrict__ cu, int S, int H, int d, int dv, int activation) {
+  extern __shared__ float lds[];
+  ChunkAt at;
+  if (!find_chunk(cu, S, blockIdx.x, at)) return;
+  const int h = blockIdx.y, n = at.count;
+  const int d16 = round16(d), dv16 = round16(dv);
+  float* Kt = lds;                          // [d16][kTokStride]
+  float* Vt = lds + d16 * kTokStride;       // [dv16][kTokStride]
+  const float l2 = log2f(decay[h]);
+  for (int idx = threadIdx.x; idx < kChunk * d16; idx += blockDim.x) {
+    const int s = idx / d16, i = idx - s * d16;
+    float val = 0.f;
+    if (s < n && i < d)
+      val = act_in(k[(long long)(at.first + s) * ldk + h * d + i], activation) *
+            exp2f(l2 * (float)(n - 1 - s));
+    Kt[i * kTokStride + s] = val;
+  }
+  for (int idx = threadIdx.x; idx < kChunk * dv16; idx += blockDim.x) {
+    const int s = idx / dv16, j = idx - s * dv16;
+    float val = 0.f;
+    if (s < n && j < dv) val = act_in(v[(long long)(at.first + s) * ldv + h * dv + j], activation);
+    Vt[j * kTokStride + s] = val;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int l16 = lane % 16, lg = lane / 16;
+  float* out = ws + ((long long)blockIdx.x * H + h) * dv * d;
+  const int iblocks = d16 / 16;
+  for (int jb = wave; jb < dv16 / 16; jb += 4) {
+    const float* a_row = Vt + (jb * 16 + l16) * kTokStride;
+    for (int ib0 = 0; ib0 < iblocks; ib0 += 4) {
+      const float* b_row[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        b_row[b] = Kt + (min(ib0 + b, iblocks - 1) * 16 + l16) * kTokStride;
+      mma_f32x4 acc[4];
+      wave_tile_product<float, 4, true>(a_row, b_row, kChunk, acc);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int i = (ib0 + b) * 16 + l16;
+        if (ib0 + b < iblocks && i < d) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = jb * 16 + 4 * lg + r;
+            if (j < dv) out[(long long)j * d + i] = acc[b][r];
+          }
+        }
+      }
+    }
+  }
+}
+
+// Every sequence's chunks in order: the chunk's entry in ws becomes the state in front of it,
+// the state moves on by S <- decay^n S + A, and the slot keeps what the last chunk leaves.  A
+// thread per state element; grid (elements / 256, sequences).
+__global__ __launch_bounds__(256) void decay_chunk_join_kernel(
+    float* __restrict__ ws, float* __restrict__ state, long long state_stride,
+    const float* __restrict__ decay, const int* __restrict__ cu, const int* __restrict__ slots,
+    int H, int d, int dv) {
+  const int s = blockIdx.y;
+  const long long per_head = (long long)dv * d, all = per_head * H;
+  const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= all) return;
+  const int len = cu[s + 1] - cu[s];
+  if (len <= 0) return;
+  int first = 0;
+  for (int p = 0; p < s; ++p) first += (cu[p + 1] - cu[p] + kChunk - 1) / kChunk;
+  const float l2 = log2f(decay[(int)(e / per_head)]);
+  const float whole = exp2f(l2 * (float)kChunk);
+  float* st = state + (long long)slots[s] * state_stride + e;
+  float cur = *st;
+  const int nc = (len + kChunk - 1) / kChunk;
+  for (int c = 0; c < nc; ++c) {
+    float* slot = ws + (long long)(first + c) * all + e;
+    const float add = *slot;
+    *slot = cur;
+    const int n = min(kChunk, len - c * kChunk);
+    cur = fmaf(n == kChunk ? whole : exp2f(l2 * (float)n), cur, add);
+  }
+  *st = cur;
+}
+
+// A chunk's read-outs from the state in front of it (ws) and from its own tokens:
+// O = (Q K^T . D) V + diag(decay^(t+1)) Q S^T with D[t][s] = decay^(t-s) for s <= t, else 0.
+// grid (chunks, heads); a wave owns 16 tokens.  STATE_ALIGNED: the state's rows take 16-byte
+// loads (d a multiple of 4).
+template <bool STATE_ALIGNED>
+__global__ __launch_bounds__(256) void decay_chunk_outputs_kernel(
+    float* __restrict__ out, const float* __restrict__ q, long long ldq,
+    const float* __restrict__ k, long long ldk, const float* __restrict__ v, long long ldv,
+    const float* __restrict__ decay, const float* __restrict__ ws, const int* __restrict__ cu,
+    int S, int H, int d, int dv, int activation) {
+  extern __shared__ float lds[];
+  ChunkAt at;
+  if (!find_chunk(cu, S, blockIdx.x, at)) return;
+  const int h = blockIdx.y, n = at.count;
+  const int d16 = round16(d), dv16 = round16(dv), DS = d16 + 4;
+  float* Qs = lds;                              // [kChunk][DS]
+  float* Ks = Qs + kChunk * DS;                 // [kChunk][DS]
+  float* Vt = Ks + kChunk * DS;                 // [dv16][kTokStride]
+  float* Ps = Vt + dv16 * kTokStride;           // [kChunk][kTokStride]
+  const float l2 = log2f(decay[h]);
+  for (int idx = threadIdx.x; idx < kChunk * d16; idx += blockDim.x) {
+    const int s = idx / d16, i = idx - s * d16;
+    const bool live = s < n && i < d;
+    const long long t = at.first + (live ? s : 0);
+    const int c = h * d + (live ? i : 0);
+    const float qv = act_in(q[t * ldq + c], activation), kv = act_in(k[t * ldk + c], activation);
+    Qs[s * DS + i] = live ? qv : 0.f;
+    Ks[s * DS + i] = live ? kv : 0.f;
+  }
+  for (int idx = threadIdx.x; idx < kChunk * dv16; idx += blockDim.x) {
+    const int s = idx / dv16, j = idx - s * dv16;
+    float val = 0.f;
+    if (s < n && j < dv) val = act_in(v[(long long)(at.first + s) * ldv + h * dv + j], activation);
+    Vt[j * kTokStride + s] = val;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int l16 = lane % 16, lg = lane / 16;
+  const float* q_row = Qs + (wave * 16 + l16) * DS;
+  {
+    const float* b_row[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) b_row[b] = Ks + (b * 16 + l16) * DS;
+    mma_f32x4 acc[4];
+    wave_tile_product<float, 4, true>(q_row, b_row, d16, acc);
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = wave * 16 + 4 * lg + r, s = b * 16 + l16;
+        Ps[t * kTokStride + s] = s <= t ? acc[b][r] * exp2f(l2 * (float)(t - s)) : 0.f;
+      }
+  }
+  __syncthreads();
+  const float* p_row = Ps + (wave * 16 + l16) * kTokStride;
+  const float* s0 = ws + ((long long)blockIdx.x * H + h) * dv * d;
+  const int jblocks = dv16 / 16;
+  float grown[4];                               // decay^(t + 1) of the lane's four tokens
+#pragma unroll
+  for (int r = 0; r < 4; ++r) grown[r] = exp2f(l2 * (float)(wave * 16 + 4 * lg + r + 1));
+  for (int jb0 = 0; jb0 < jblocks; jb0 += 4) {
+    const float* v_row[4];
+    const float* s_row[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int jb = min(jb0 + b, jblocks - 1);
+      v_row[b] = Vt + (jb * 16 + l16) * kTokStride;
+      s_row[b] = s0 + (long long)min(jb * 16 + l16, dv - 1) * d;
+    }
+    mma_f32x4 own[4], carried[4];
+    wave_tile_product<float, 4, true>(p_row, v_row, kChunk, own);
+    wave_tile_product<float, 4, STATE_ALIGNED>(q_row, s_row, d, carried);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int j = (jb0 + b) * 16 + l16;
+      if (jb0 + b < jblocks && j < dv) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = wave * 16 + 4 * lg + r;
+          if (t < n)
+            out[(long long)(at.first + t) * H * dv + h * dv + j] =
+                fmaf(grown[r], carried[b][r], own[b][r]);
+        }
+      }
+    }
+  }
+}
+
+// More dynamic LDS than a kernel gets unasked, asked for once on every device.
+static int grant_lds(const void* kernel, size_t bytes, bool* granted) {
+  constexpr int kDevices = 64;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return 1;
+  if (dev >= 0 && dev < kDevices && granted[dev]) return 0;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) return 1;
+  if (dev >= 0 && dev < kDevices) granted[dev] = true;
+  return 0;
+}
+
 }  // namespace
 
 // out (T, H * dv) float32; q, k (T, >= H * d) and v (T, >= H * dv) with row strides, float32 or
@@ -140,5 +364,58 @@ RLIS_API int rlis_decay_attention_scan(float* out, const void* q, long long ldq,
 #undef BY_KR
 #undef LAUNCH
   RLIS_LAUNCH_CHECK("decay_attention_scan");
+  return 0;
+}
+
+// The same result as rlis_decay_attention_scan (to rounding) for steps of long portions, in
+// three launches: every chunk of 64 tokens from a zero state, the chunks of a sequence joined in
+// order, every chunk's read-outs.  q, k, v float32; d and dv at most 128; ws: (max_chunks, H,
+// dv, d) floats with max_chunks at least the step's chunks (T / 64 + S bounds them).
+RLIS_API int rlis_decay_attention_chunks(float* out, const float* q, long long ldq,
+                                         const float* k, long long ldk, const float* v,
+                                         long long ldv, const float* decay, float* state,
+                                         long long state_stride, const int* cu, const int* slots,
+                                         int S, int T, int H, int d, int dv, int activation,
+                                         float* ws, int max_chunks, hipStream_t stream) {
+  RLIS_REQUIRE(S >= 0 && T >= 0 && H > 0 && d > 0 && dv > 0,
+               "decay_attention_chunks: bad sizes S=%d T=%d H=%d d=%d dv=%d", S, T, H, d, dv);
+  RLIS_REQUIRE(d <= 128 && dv <= 128,
+               "decay_attention_chunks: heads of %d and %d channels, at most 128", d, dv);
+  RLIS_REQUIRE(H <= 65535 && S <= 65535, "decay_attention_chunks: too many heads or sequences");
+  RLIS_REQUIRE(ldq >= (long long)H * d && ldk >= (long long)H * d && ldv >= (long long)H * dv,
+               "decay_attention_chunks: row strides shorter than the heads");
+  RLIS_REQUIRE(state_stride >= (long long)H * dv * d, "decay_attention_chunks: state too short");
+  RLIS_REQUIRE(ws && max_chunks >= T / kChunk + S,
+               "decay_attention_chunks: workspace of %d chunks for %d tokens of %d sequences",
+               max_chunks, T, S);
+  if (S == 0 || T == 0) return 0;
+  const int d16 = (d + 15) / 16 * 16, dv16 = (dv + 15) / 16 * 16;
+  const size_t lds_states = (size_t)(d16 + dv16) * kTokStride * sizeof(float);
+  const size_t lds_outputs =
+      ((size_t)2 * kChunk * (d16 + 4) + (size_t)(dv16 + kChunk) * kTokStride) * sizeof(float);
+  static bool granted[3][64];
+  constexpr size_t kMostLds = 160 * 1024;
+  RLIS_REQUIRE(lds_outputs <= kMostLds, "decay_attention_chunks: %zu bytes of LDS", lds_outputs);
+  const bool aligned = d % 4 == 0 && ((uintptr_t)ws % 16 == 0);
+  RLIS_REQUIRE(
+      grant_lds(reinterpret_cast<const void*>(&decay_chunk_states_kernel), kMostLds, granted[0]) == 0 &&
+      grant_lds(reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<true>), kMostLds, granted[1]) == 0 &&
+      grant_lds(reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<false>), kMostLds, granted[2]) == 0,
+      "decay_attention_chunks: the device grants no %zu bytes of LDS", kMostLds);
+  const dim3 grid(max_chunks, H);
+  decay_chunk_states_kernel<<<grid, 256, lds_states, stream>>>(ws, k, ldk, v, ldv, decay, cu, S, H,
+                                                               d, dv, activation);
+  RLIS_LAUNCH_CHECK("decay_attention_chunks (states)");
+  const long long elements = (long long)H * dv * d;
+  decay_chunk_join_kernel<<<dim3((unsigned)((elements + 255) / 256), S), 256, 0, stream>>>(
+      ws, state, state_stride, decay, cu, slots, H, d, dv);
+  RLIS_LAUNCH_CHECK("decay_attention_chunks (join)");
+  if (aligned)
+    decay_chunk_outputs_kernel<true><<<grid, 256, lds_outputs, stream>>>(
+        out, q, ldq, k, ldk, v, ldv, decay, ws, cu, S, H, d, dv, activation);
+  else
+    decay_chunk_outputs_kernel<false><<<grid, 256, lds_outputs, stream>>>(
+        out, q, ldq, k, ldk, v, ldv, decay, ws, cu, S, H, d, dv, activation);
+  RLIS_LAUNCH_CHECK("decay_attention_chunks (outputs)");
   return 0;
 }

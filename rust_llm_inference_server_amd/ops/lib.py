@@ -21,6 +21,7 @@ _SIGNATURES = {
     "rlis_gelu_tanh": [P, P, I, L, P],
     "rlis_depth_mix": [P, P, P, L, I, P, I, I, P],
     "rlis_decay_attention_scan": [P, P, L, P, L, P, L, I, P, P, L, P, P, I, I, I, I, I, I, P],
+    "rlis_decay_attention_chunks": [P, P, L, P, L, P, L, P, P, L, P, P, I, I, I, I, I, I, P, I, P],
     "rlis_add_residual": [P, P, I, L, I, I, F, P],
     "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
     "rlis_swiglu": [P, P, I, I, I, P],
@@ -61,9 +62,9 @@ _SIGNATURES = {
     "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P, F, P],
     "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P, F, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, I, I, I,
-                              P, P, I, P, P, L, L, P, P],
+                              P, P, I, P, P, L, L, P, P, F, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,
-                               P, P, I, P, P],
+                               P, P, I, P, P, F, P],
     "rlis_attn_reduce_rows": [P, L, P, P, P, P, I, I, I, I, I, P],
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
     "rlis_fill_normal_device": [P, I, L, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_double,

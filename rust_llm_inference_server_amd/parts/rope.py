@@ -25,8 +25,8 @@ def yarn_frequencies(rot_dim: int, theta: float, scaling: Dict[str, Any]) -> tor
     ``rot_dim ln(original / (2 pi n)) / (2 ln theta)``: pairs up to ``lo = floor(turns(fast))``
     keep ``f_i = theta^(-2 i / rot_dim)``, pairs from ``hi = ceil(turns(slow))`` on get
     ``f_i / factor``, and between the two the share of the stretched frequency rises linearly."""
-    factor, original = float(scaling["factor"]), float(scaling["original"])
-    fast, slow = float(scaling["fast"]), float(scaling["slow"])
+    factor, original, fast, slow = (float(scaling.get(key) or 0.0)
+                                    for key in ("factor", "original", "fast", "slow"))
     if not (factor > 0 and original > 0 and fast > 0 and slow > 0):
         raise ValueError("position encoding 'rope': yarn scaling needs positive 'factor', "
                          "'original', 'fast' and 'slow'")

@@ -55,6 +55,9 @@ def test_position_part_tables():
     torch.testing.assert_close(rope.sin.cpu(), sin, atol=1e-6, rtol=0)
     with pytest.raises(ValueError, match="unknown scaling"):
         create("position", PartSpec("rope", {"rot_dim": 32, "theta": 1e4,
+                                             "scaling": {"rope_type": "ntk"}}), "", ctx_for({}))
+    with pytest.raises(ValueError, match="yarn scaling needs"):
+        create("position", PartSpec("rope", {"rot_dim": 32, "theta": 1e4,
                                              "scaling": {"rope_type": "yarn"}}), "", ctx_for({}))
 
 
