@@ -46,7 +46,10 @@ prompts, each with the bytes a step has to read (weights once, the live requests
 for Gipotar their state slots read and written) as a fraction of the HBM rate.
 ``--design bekunex`` (or ``gipotar,bekunex``) times the Bekunex design that way (attention over
 a cached latent, selective scan, a routed feed-forward; of the experts' weights a step counts
-those that its tokens reach on average, and of a windowed cache the window)."""
+those that its tokens reach on average, and of a windowed cache the window).
+``--design lagedra`` times the Lagedra design (three layers of linear attention with a fixed
+decay per head to one of windowed softmax attention behind short convolutions, feed-forwards
+that alternate between a routed mixture and a dense GELU unit)."""
 import argparse
 import copy
 import json
@@ -242,6 +245,38 @@ def bekunex_like(cfg: dict) -> dict:
             "norm": {"eps": 1e-5}, "logit_scale": 1.0, "layers": layers}
 
 
+def lagedra_like(cfg: dict) -> dict:
+    """A Lagedra configuration at the sizes of a Llama preset: the same width, depth, vocabulary,
+    heads and head size; of every four layers three are linear attention with a fixed decay per
+    head and one is windowed softmax attention (window 1,024, four taps, capped scores, rotation
+    with stretched frequencies, values mixed with the first such layer's); feed-forwards
+    alternate between a mixture of 32 bounded gated units (a quarter of the preset's
+    feed-forward width each, four chosen out of two of four groups) and a dense GELU unit of
+    one and a half times the preset's width: as many active feed-forward weights per token as
+    the preset has."""
+    W, d, H = cfg["hidden_size"], cfg["head_dim"], cfg["num_attention_heads"]
+    ff = cfg["intermediate_size"]
+    moe = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0},
+           "router": {"experts": 32, "groups": {"count": 4, "keep": 2}, "top": 4}}
+    dense = {"kind": "dense", "ff": ff * 3 // 2}
+    lightning = {"heads": H, "dim": d, "vdim": d,
+                 "decay": [1.0 - 2.0 ** -(3.0 + 6.0 * h / H) for h in range(H)]}
+    attention = {"heads": H, "kv_heads": cfg["num_key_value_heads"], "dim": d, "vdim": d,
+                 "conv": 4, "mask": {"size": 1024}, "scale": d ** -0.5, "softcap": 30.0,
+                 "v_mix": True,
+                 "rot": {"dims": d, "base": cfg["rope_theta"],
+                         "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    layers = []
+    for i in range(cfg["num_hidden_layers"]):
+        softmax = i % 4 == 3
+        layers.append(copy.deepcopy({"type": "attention" if softmax else "lightning",
+                                     "mixer": attention if softmax else lightning,
+                                     "mlp": moe if i % 2 == 0 else dense}))
+    return {"architecture": "Lagedra", "vocab": cfg["vocab_size"], "width": W,
+            "max_positions": cfg["max_position_embeddings"], "norm": {"eps": 1e-6},
+            "layers": layers}
+
+
 def step_bytes_of(model, batch: int, mean_context: float) -> float:
     """What a decode step of any model has to move: every tensor its parts hold once (the
     embedding table only where the head shares it), each live request's cached positions, and
@@ -348,7 +383,7 @@ def compare_designs(args) -> int:
             base["num_hidden_layers"] = args.layers
         longest = max(T, args.points_context + new + warm + 16) + 64
         base["max_position_embeddings"] = min(base["max_position_embeddings"], longest)
-        like = {"gipotar": gipotar_like, "bekunex": bekunex_like}
+        like = {"gipotar": gipotar_like, "bekunex": bekunex_like, "lagedra": lagedra_like}
         for design, cfg in [("llama", base)] + [(d, like[d](base)) for d in args.design.split(",")]:
             vocab = base["vocab_size"]
             model = random_model(cfg, seed=0, dtype=args.dtype, max_positions=longest)
@@ -410,7 +445,7 @@ def main() -> int:
                     help="time the Gipotar design beside the Llama presets of --sizes instead")
     ap.add_argument("--design", default="gipotar",
                     help="the designs that --designs times beside Llama, with commas between "
-                         "them: gipotar, bekunex")
+                         "them: gipotar, bekunex, lagedra")
     ap.add_argument("--sizes", default="llama-3.2-1b,llama-3.2-3b",
                     help="presets whose sizes the two designs of --designs are built at")
     args = ap.parse_args()

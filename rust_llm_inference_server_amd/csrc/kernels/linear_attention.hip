@@ -138,50 +138,93 @@ __device__ __forceinline__ bool find_chunk(const int* __restrict__ cu, int S, in
   return false;
 }
 
+// A wave's tile of a product on the float32 matrix cores for operands that lie in LDS with any
+// stride along k: C[i][n] = sum_k A[i][k] B[n][k] for 16 rows of A and NB blocks of 16 rows of
+// B.  Every lane hands in the address of element k = 0 of the row it serves (row lane % 16 of A
+// and of each block of B) and the distance between consecutive k.  The result's layout is that
+// of wave_tile_product; K is a multiple of 4.
+template <int NB>
+__device__ __forceinline__ void wave_tile_product_strided(const float* a_lane, int a_kstride,
+                                                          const float* const (&b_lane)[NB],
+                                                          int b_kstride, int K,
+                                                          mma_f32x4 (&acc)[NB]) {
+  const int g = (threadIdx.x % kWave) / 16;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) acc[b] = mma_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int k0 = 0; k0 < K; k0 += 4) {
+    const float av = a_lane[(k0 + g) * a_kstride];
+    float bv[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) bv[b] = b_lane[b][(k0 + g) * b_kstride];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+      acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv[b], acc[b], 0, 0, 0);
+  }
+}
+
+// Rows first .. first + n - 1 of a projection (columns col0 .. col0 + width - 1, through the
+// activation) into LDS as [token][channel], four channels a thread; rows from n on and
+// channels from width to width16 are zeros.  VEC: 16-byte loads (width a multiple of 4, rows
+// aligned).  l2 != 0 or weigh: row s is multiplied by 2^(l2 * (n - 1 - s)).
+template <bool VEC>
+__device__ __forceinline__ void fill_rows(float* dst, int dst_stride, const float* __restrict__ src,
+                                          long long ld, int col0, int width, int width16,
+                                          int first, int n, int activation, bool weigh, float l2) {
+  const int groups = width16 / 4;
+  for (int idx = threadIdx.x; idx < kChunk * groups; idx += blockDim.x) {
+    const int s = idx / groups, i = (idx - s * groups) * 4;
+    float val[4] = {0.f, 0.f, 0.f, 0.f};
+    if (s < n && i < width) {
+      const float* p = src + (long long)(first + s) * ld + col0 + i;
+      if (VEC) {
+        const mma_f32x4 v = *reinterpret_cast<const mma_f32x4*>(p);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) val[c] = v[c];
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) val[c] = i + c < width ? p[c] : 0.f;
+      }
+      const float w = weigh ? exp2f(l2 * (float)(n - 1 - s)) : 1.0f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) val[c] = i + c < width ? act_in(val[c], activation) * w : 0.f;
+    }
+    *reinterpret_cast<mma_f32x4*>(dst + s * dst_stride + i) =
+        mma_f32x4{val[0], val[1], val[2], val[3]};
+  }
+}
+
 // What a chunk of n tokens adds to the state, from a zero state: A[j][i] = sum_s decay^(n-1-s)
-// k_s[i] v_s[j], the product over the tokens of V^T and of K^T with the decays folded in, both
-// transposed into LDS.  grid (chunks, heads); ws holds (chunk, head, value channel, key
-// channel).
+// k_s[i] v_s[j], the product over the tokens of V and of K with the decays folded in, both in
+// LDS as they come ([token][channel]).  grid (chunks, heads); ws holds (chunk, head, value
+// channel, key channel).
+template <bool VEC>
 __global__ __launch_bounds__(256) void decay_chunk_states_kernel(
     float* __restrict__ ws, const float* __restrict__ k, long long ldk,
     const float* __restrict__ v, long long ldv, const float* __restrict__ decay,
     const int* __restrict__ cu, int S, int H, int d, int dv, int activation) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   ChunkAt at;
   if (!find_chunk(cu, S, blockIdx.x, at)) return;
   const int h = blockIdx.y, n = at.count;
-  const int d16 = round16(d), dv16 = round16(dv);
-  float* Kt = lds;                          // [d16][kTokStride]
-  float* Vt = lds + d16 * kTokStride;       // [dv16][kTokStride]
-  const float l2 = log2f(decay[h]);
-  for (int idx = threadIdx.x; idx < kChunk * d16; idx += blockDim.x) {
-    const int s = idx / d16, i = idx - s * d16;
-    float val = 0.f;
-    if (s < n && i < d)
-      val = act_in(k[(long long)(at.first + s) * ldk + h * d + i], activation) *
-            exp2f(l2 * (float)(n - 1 - s));
-    Kt[i * kTokStride + s] = val;
-  }
-  for (int idx = threadIdx.x; idx < kChunk * dv16; idx += blockDim.x) {
-    const int s = idx / dv16, j = idx - s * dv16;
-    float val = 0.f;
-    if (s < n && j < dv) val = act_in(v[(long long)(at.first + s) * ldv + h * dv + j], activation);
-    Vt[j * kTokStride + s] = val;
-  }
+  const int d16 = round16(d), dv16 = round16(dv), DS = d16 + 4, DVS = dv16 + 4;
+  float* Ks = lds;                          // [kChunk][DS]
+  float* Vs = lds + kChunk * DS;            // [kChunk][DVS]
+  fill_rows<VEC>(Ks, DS, k, ldk, h * d, d, d16, at.first, n, activation, true, log2f(decay[h]));
+  fill_rows<VEC>(Vs, DVS, v, ldv, h * dv, dv, dv16, at.first, n, activation, false, 0.f);
   __syncthreads();
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int l16 = lane % 16, lg = lane / 16;
   float* out = ws + ((long long)blockIdx.x * H + h) * dv * d;
   const int iblocks = d16 / 16;
   for (int jb = wave; jb < dv16 / 16; jb += 4) {
-    const float* a_row = Vt + (jb * 16 + l16) * kTokStride;
+    const float* a_lane = Vs + jb * 16 + l16;
     for (int ib0 = 0; ib0 < iblocks; ib0 += 4) {
-      const float* b_row[4];
+      const float* b_lane[4];
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
-        b_row[b] = Kt + (min(ib0 + b, iblocks - 1) * 16 + l16) * kTokStride;
+      for (int b = 0; b < 4; ++b) b_lane[b] = Ks + min(ib0 + b, iblocks - 1) * 16 + l16;
       mma_f32x4 acc[4];
-      wave_tile_product<float, 4, true>(a_row, b_row, kChunk, acc);
+      wave_tile_product_strided<4>(a_lane, DVS, b_lane, DS, kChunk, acc);
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         const int i = (ib0 + b) * 16 + l16;
@@ -229,39 +272,27 @@ __global__ __launch_bounds__(256) void decay_chunk_join_kernel(
 
 // A chunk's read-outs from the state in front of it (ws) and from its own tokens:
 // O = (Q K^T . D) V + diag(decay^(t+1)) Q S^T with D[t][s] = decay^(t-s) for s <= t, else 0.
-// grid (chunks, heads); a wave owns 16 tokens.  STATE_ALIGNED: the state's rows take 16-byte
-// loads (d a multiple of 4).
-template <bool STATE_ALIGNED>
+// grid (chunks, heads); a wave owns 16 tokens.  VEC: 16-byte loads of the inputs;
+// STATE_ALIGNED: the state's rows take 16-byte loads (d a multiple of 4).
+template <bool VEC, bool STATE_ALIGNED>
 __global__ __launch_bounds__(256) void decay_chunk_outputs_kernel(
     float* __restrict__ out, const float* __restrict__ q, long long ldq,
     const float* __restrict__ k, long long ldk, const float* __restrict__ v, long long ldv,
     const float* __restrict__ decay, const float* __restrict__ ws, const int* __restrict__ cu,
     int S, int H, int d, int dv, int activation) {
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   ChunkAt at;
   if (!find_chunk(cu, S, blockIdx.x, at)) return;
   const int h = blockIdx.y, n = at.count;
-  const int d16 = round16(d), dv16 = round16(dv), DS = d16 + 4;
+  const int d16 = round16(d), dv16 = round16(dv), DS = d16 + 4, DVS = dv16 + 4;
   float* Qs = lds;                              // [kChunk][DS]
   float* Ks = Qs + kChunk * DS;                 // [kChunk][DS]
-  float* Vt = Ks + kChunk * DS;                 // [dv16][kTokStride]
-  float* Ps = Vt + dv16 * kTokStride;           // [kChunk][kTokStride]
+  float* Vs = Ks + kChunk * DS;                 // [kChunk][DVS]
+  float* Ps = Vs + kChunk * DVS;                // [kChunk][kTokStride]
   const float l2 = log2f(decay[h]);
-  for (int idx = threadIdx.x; idx < kChunk * d16; idx += blockDim.x) {
-    const int s = idx / d16, i = idx - s * d16;
-    const bool live = s < n && i < d;
-    const long long t = at.first + (live ? s : 0);
-    const int c = h * d + (live ? i : 0);
-    const float qv = act_in(q[t * ldq + c], activation), kv = act_in(k[t * ldk + c], activation);
-    Qs[s * DS + i] = live ? qv : 0.f;
-    Ks[s * DS + i] = live ? kv : 0.f;
-  }
-  for (int idx = threadIdx.x; idx < kChunk * dv16; idx += blockDim.x) {
-    const int s = idx / dv16, j = idx - s * dv16;
-    float val = 0.f;
-    if (s < n && j < dv) val = act_in(v[(long long)(at.first + s) * ldv + h * dv + j], activation);
-    Vt[j * kTokStride + s] = val;
-  }
+  fill_rows<VEC>(Qs, DS, q, ldq, h * d, d, d16, at.first, n, activation, false, 0.f);
+  fill_rows<VEC>(Ks, DS, k, ldk, h * d, d, d16, at.first, n, activation, false, 0.f);
+  fill_rows<VEC>(Vs, DVS, v, ldv, h * dv, dv, dv16, at.first, n, activation, false, 0.f);
   __syncthreads();
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int l16 = lane % 16, lg = lane / 16;
@@ -288,16 +319,17 @@ __global__ __launch_bounds__(256) void decay_chunk_outputs_kernel(
 #pragma unroll
   for (int r = 0; r < 4; ++r) grown[r] = exp2f(l2 * (float)(wave * 16 + 4 * lg + r + 1));
   for (int jb0 = 0; jb0 < jblocks; jb0 += 4) {
-    const float* v_row[4];
+    const float* v_lane[4];
     const float* s_row[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const int jb = min(jb0 + b, jblocks - 1);
-      v_row[b] = Vt + (jb * 16 + l16) * kTokStride;
+      v_lane[b] = Vs + jb * 16 + l16;
       s_row[b] = s0 + (long long)min(jb * 16 + l16, dv - 1) * d;
     }
     mma_f32x4 own[4], carried[4];
-    wave_tile_product<float, 4, true>(p_row, v_row, kChunk, own);
+    // (a wave's tokens see the keys up to its own last one)
+    wave_tile_product_strided<4>(p_row, 1, v_lane, DVS, (wave + 1) * 16, own);
     wave_tile_product<float, 4, STATE_ALIGNED>(q_row, s_row, d, carried);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -390,32 +422,45 @@ RLIS_API int rlis_decay_attention_chunks(float* out, const float* q, long long l
                max_chunks, T, S);
   if (S == 0 || T == 0) return 0;
   const int d16 = (d + 15) / 16 * 16, dv16 = (dv + 15) / 16 * 16;
-  const size_t lds_states = (size_t)(d16 + dv16) * kTokStride * sizeof(float);
+  const size_t lds_states = (size_t)kChunk * (d16 + dv16 + 8) * sizeof(float);
   const size_t lds_outputs =
-      ((size_t)2 * kChunk * (d16 + 4) + (size_t)(dv16 + kChunk) * kTokStride) * sizeof(float);
-  static bool granted[3][64];
+      (size_t)kChunk * (2 * (d16 + 4) + dv16 + 4 + kTokStride) * sizeof(float);
   constexpr size_t kMostLds = 160 * 1024;
   RLIS_REQUIRE(lds_outputs <= kMostLds, "decay_attention_chunks: %zu bytes of LDS", lds_outputs);
+  const bool vec = d % 4 == 0 && dv % 4 == 0 && ldq % 4 == 0 && ldk % 4 == 0 && ldv % 4 == 0 &&
+                   (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0;
   const bool aligned = d % 4 == 0 && ((uintptr_t)ws % 16 == 0);
-  RLIS_REQUIRE(
-      grant_lds(reinterpret_cast<const void*>(&decay_chunk_states_kernel), kMostLds, granted[0]) == 0 &&
-      grant_lds(reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<true>), kMostLds, granted[1]) == 0 &&
-      grant_lds(reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<false>), kMostLds, granted[2]) == 0,
-      "decay_attention_chunks: the device grants no %zu bytes of LDS", kMostLds);
+  static bool granted[6][64];
+  const void* kernels[6] = {
+      reinterpret_cast<const void*>(&decay_chunk_states_kernel<true>),
+      reinterpret_cast<const void*>(&decay_chunk_states_kernel<false>),
+      reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<true, true>),
+      reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<false, true>),
+      reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<true, false>),
+      reinterpret_cast<const void*>(&decay_chunk_outputs_kernel<false, false>)};
+  for (int i = 0; i < 6; ++i)
+    RLIS_REQUIRE(grant_lds(kernels[i], kMostLds, granted[i]) == 0,
+                 "decay_attention_chunks: the device grants no %zu bytes of LDS", kMostLds);
   const dim3 grid(max_chunks, H);
-  decay_chunk_states_kernel<<<grid, 256, lds_states, stream>>>(ws, k, ldk, v, ldv, decay, cu, S, H,
-                                                               d, dv, activation);
+  if (vec)
+    decay_chunk_states_kernel<true><<<grid, 256, lds_states, stream>>>(ws, k, ldk, v, ldv, decay,
+                                                                      cu, S, H, d, dv, activation);
+  else
+    decay_chunk_states_kernel<false><<<grid, 256, lds_states, stream>>>(ws, k, ldk, v, ldv, decay,
+                                                                       cu, S, H, d, dv, activation);
   RLIS_LAUNCH_CHECK("decay_attention_chunks (states)");
   const long long elements = (long long)H * dv * d;
   decay_chunk_join_kernel<<<dim3((unsigned)((elements + 255) / 256), S), 256, 0, stream>>>(
       ws, state, state_stride, decay, cu, slots, H, d, dv);
   RLIS_LAUNCH_CHECK("decay_attention_chunks (join)");
-  if (aligned)
-    decay_chunk_outputs_kernel<true><<<grid, 256, lds_outputs, stream>>>(
-        out, q, ldq, k, ldk, v, ldv, decay, ws, cu, S, H, d, dv, activation);
-  else
-    decay_chunk_outputs_kernel<false><<<grid, 256, lds_outputs, stream>>>(
-        out, q, ldq, k, ldk, v, ldv, decay, ws, cu, S, H, d, dv, activation);
+#define OUTPUTS(V_, A_)                                                          \
+  decay_chunk_outputs_kernel<V_, A_><<<grid, 256, lds_outputs, stream>>>(        \
+      out, q, ldq, k, ldk, v, ldv, decay, ws, cu, S, H, d, dv, activation)
+  if (vec && aligned) OUTPUTS(true, true);
+  else if (vec) OUTPUTS(true, false);
+  else if (aligned) OUTPUTS(false, true);
+  else OUTPUTS(false, false);
+#undef OUTPUTS
   RLIS_LAUNCH_CHECK("decay_attention_chunks (outputs)");
   return 0;
 }

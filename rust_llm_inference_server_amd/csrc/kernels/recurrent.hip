@@ -808,6 +808,31 @@ __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(
   }
 }
 
+// The same for heads of many channels (the norm over all the heads together): a workgroup of
+// four waves per (token, head), their sums of squares joined through LDS in a fixed order.
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void head_norm_gate_wide_kernel(
+    TO* __restrict__ out, const float* __restrict__ o, const float* __restrict__ weight,
+    int weight_stride, const TG* __restrict__ gate, long long ldg, int heads, int dv, float eps,
+    int sigmoid_gate) {
+  __shared__ float partial[4];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* row = o + ((long long)t * heads + h) * dv;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < dv; j += 256) ss += row[j] * row[j];
+  ss = wave_sum(ss);
+  if (threadIdx.x % kWave == 0) partial[threadIdx.x / kWave] = ss;
+  __syncthreads();
+  ss = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+  const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+  for (int j = threadIdx.x; j < dv; j += 256) {
+    const float g = ld(gate + (long long)t * ldg + h * dv + j);
+    st(out + ((long long)t * heads + h) * dv + j,
+       row[j] * inv * weight[h * weight_stride + j] *
+           (sigmoid_gate ? 1.0f / (1.0f + expf(-g)) : siluf_(g)));
+  }
+}
+
 }  // namespace
 
 // ============================================================================ entry points
@@ -996,11 +1021,17 @@ RLIS_API int rlis_head_norm_gate(void* out, int out_dtype, const float* o, const
   if (T == 0) return 0;
   const dim3 grid(T, heads);
   const int key = gate_dtype * 2 + out_dtype;
+  const bool wide = dv >= 512;       // (by the head's size alone: a row's sums do not depend on the batch)
 #define CASE(k_, TG, TO)                                                                     \
   case k_:                                                                                   \
-    head_norm_gate_kernel<TG, TO><<<grid, kWave, 0, stream>>>(                               \
-        (TO*)out, o, weight, weight_stride, (const TG*)gate, ldg, heads, dv, eps,            \
-        sigmoid_gate);                                                                       \
+    if (wide)                                                                                \
+      head_norm_gate_wide_kernel<TG, TO><<<grid, 256, 0, stream>>>(                          \
+          (TO*)out, o, weight, weight_stride, (const TG*)gate, ldg, heads, dv, eps,          \
+          sigmoid_gate);                                                                     \
+    else                                                                                     \
+      head_norm_gate_kernel<TG, TO><<<grid, kWave, 0, stream>>>(                             \
+          (TO*)out, o, weight, weight_stride, (const TG*)gate, ldg, heads, dv, eps,          \
+          sigmoid_gate);                                                                     \
     break;
   switch (key) {
     CASE(0, float, float)
