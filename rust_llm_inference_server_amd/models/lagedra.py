@@ -81,6 +81,8 @@ def lagedra_spec(cfg: LagedraConfig) -> ModelSpec:
         layers.append(LayerSpec(block, f"l{i}"))
         if ff is None:
             optional.append(f"l{i}.norm2")
+        if layer.type == "attention" and not layer.mixer.v_mix:
+            optional.append(f"l{i}.mix.vmix")       # may be stored, is not read
     return ModelSpec(
         hidden_size=W,
         vocab_size=cfg.vocab,
