@@ -265,7 +265,7 @@ def lagedra_like(cfg: dict) -> dict:
                  "conv": 4, "mask": {"size": 1024}, "scale": d ** -0.5, "softcap": 30.0,
                  "v_mix": True,
                  "rot": {"dims": d, "base": cfg["rope_theta"],
-                         "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+                         "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
     layers = []
     for i in range(cfg["num_hidden_layers"]):
         softmax = i % 4 == 3

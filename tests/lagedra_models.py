@@ -53,7 +53,7 @@ CONFIG_A = {
         _attention(4, 2, 16, 24, 3, 20, 8, 1000.0, (4.0, 64, 8.0, 1.0), 0.3, 6.0, False,
                    _dense(72)),
         _lightning(3, 24, 40, [0.5, 0.9, 0.999], _moe(24, 1.5, 6, 3, 2, 2)),
-        _attention(6, 2, 8, 12, 2, 16, 8, 50000.0, None, 0.4, 4.0, True, None),
+        _attention(6, 2, 8, 12, 2, 16, 8, 40000.0, None, 0.4, 4.0, True, None),
         _lightning(2, 16, 8, [1.0, 0.7], _dense(40)),
         _attention(2, 2, 24, 12, 4, 33, 16, 300.0, (2.0, 32, 4.0, 0.5), 0.25, 9.0, True,
                    _moe(16, 0.7, 4, 1, 1, 1)),
@@ -84,7 +84,23 @@ CONFIG_C = {
                    _dense(30)),
     ],
 }
-CONFIGS = {"a": CONFIG_A, "b": CONFIG_B, "c": CONFIG_C}
+# Head sizes that the matrix-core kernels take as they are (64 with the whole head rotated, which
+# the attention kernels can do themselves; 128 and 32 for keys and values with half the head
+# rotated; 48 and 64, padded to one size), heads of 64 and 128 channels in the linear attention,
+# for prompts of hundreds of tokens.
+CONFIG_D = {
+    "architecture": "Lagedra", "vocab": 200, "width": 128, "max_positions": 1024,
+    "norm": {"eps": 1e-6},
+    "layers": [
+        _lightning(2, 64, 64, [0.9, 0.995], _dense(192)),
+        _attention(4, 2, 64, 64, 3, 100, 64, 10000.0, (8.0, 256, 16.0, 2.0), 0.125, 15.0, True,
+                   _moe(64, 1.0, 8, 2, 1, 2)),
+        _lightning(1, 128, 128, [0.98], _moe(32, 2.0, 4, 2, 2, 3)),
+        _attention(2, 1, 128, 32, 4, 40, 64, 500000.0, None, 0.09, 25.0, False, _dense(160)),
+        _attention(4, 2, 48, 64, 2, 300, 48, 20000.0, (2.0, 512, 8.0, 1.0), 0.14, 10.0, True, None),
+    ],
+}
+CONFIGS = {"a": CONFIG_A, "b": CONFIG_B, "c": CONFIG_C, "d": CONFIG_D}
 
 
 def spec_of(config: dict):

@@ -233,6 +233,25 @@ def test_long_prompts_and_long_decoding(backend, dtype, name, tmp_path_factory):
     check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
 
 
+def test_prompts_of_hundreds_of_tokens_at_head_sizes_of_real_models(backend, dtype,
+                                                                    tmp_path_factory):
+    """Heads of 64 and 128: whole prompts of up to 700 tokens in one step (the linear
+    attention's chunks, the attention kernels' tiles of 64 and 128 queries, the rotation inside
+    the attention kernel where the whole head of 64 turns), the same prompts with their ends
+    decoded, and in portions beside each other."""
+    folder, cfg, stored = model_case("d", dtype, tmp_path_factory)
+    lengths = [300, 130] if backend.type == "cpu" else [700, 300, 130, 257]
+    reqs = traces.random_requests(cfg["vocab"], lengths, seed=71)
+    make = lambda: runner_for(folder, backend, dtype, num_pages=130, max_positions=1024)
+    steps, _ = traces.trace_whole(reqs)
+    check_trace(make(), steps, reqs, cfg, stored, dtype)
+    steps, _ = traces.trace_tail(reqs, tail=20)
+    check_trace(make(), steps, reqs, cfg, stored, dtype)
+    steps, peak = traces.trace_mixed(reqs, live=3, seed=6)
+    check_trace(runner_for(folder, backend, dtype, num_pages=-(-peak // 16), max_num_seqs=3,
+                           max_positions=1024), steps, reqs, cfg, stored, dtype)
+
+
 # ------------------------------------------------------------- keys made to stand out
 KEY_TOKEN, QUERY_TOKEN, FILL_TOKEN = 5, 9, 1
 
