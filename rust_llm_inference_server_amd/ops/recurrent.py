@@ -235,32 +235,39 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, he
 
 
 # A step of at least DECAY_CHUNKED_MIN_TOKENS tokens whose sequences bring at least
-# DECAY_CHUNKED_MIN_MEAN_TOKENS each on average takes the chunked form of the linear attention
-# (chunks of DECAY_CHUNK_LEN tokens on the matrix cores, float32 products; heads of at most
-# DECAY_CHUNKED_MAX_DIM channels); every other step walks token by token.  The two agree to
-# rounding.  The rule looks at what the host knows: rows and sequences of the step.
+# DECAY_CHUNKED_MIN_MEAN_TOKENS each on average, or any step in which one sequence brings
+# DECAY_CHUNKED_MIN_TOKENS (a long portion beside decoded tokens), takes the chunked form of the
+# linear attention (chunks of DECAY_CHUNK_LEN tokens on the matrix cores, float32 products; heads
+# of at most DECAY_CHUNKED_MAX_DIM channels); every other step walks token by token.  The two
+# agree to rounding.  The rule looks at what the host knows: rows and sequences of the step and
+# its longest portion.
 DECAY_CHUNKED_MIN_TOKENS = 256
 DECAY_CHUNKED_MIN_MEAN_TOKENS = 64
 DECAY_CHUNKED_MAX_DIM = 128
 DECAY_CHUNK_LEN = 64
 
 
-def decay_attention_chunked(T: int, num_seqs: int, dim: int, vdim: int, dtype: torch.dtype) -> bool:
-    return (dtype == torch.float32 and max(dim, vdim) <= DECAY_CHUNKED_MAX_DIM
-            and T >= DECAY_CHUNKED_MIN_TOKENS
+def decay_attention_chunked(T: int, num_seqs: int, dim: int, vdim: int, dtype: torch.dtype,
+                            longest: Optional[int] = None) -> bool:
+    if dtype != torch.float32 or max(dim, vdim) > DECAY_CHUNKED_MAX_DIM:
+        return False
+    if longest is not None and longest >= DECAY_CHUNKED_MIN_TOKENS:
+        return True
+    return (T >= DECAY_CHUNKED_MIN_TOKENS
             and T >= DECAY_CHUNKED_MIN_MEAN_TOKENS * max(1, num_seqs))
 
 
 def decay_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor,
                     state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
-                    heads: int, dim: int, vdim: int, activation: bool = True) -> torch.Tensor:
+                    heads: int, dim: int, vdim: int, activation: bool = True,
+                    longest: Optional[int] = None) -> torch.Tensor:
     """Linear attention with a fixed decay per head: ``S <- decay[h] S + k v^T``, ``o = S^T q``
     (the token's own key and value are in what its query reads).  ``q``, ``k`` ``(T, heads *
     dim)`` and ``v`` ``(T, heads * vdim)`` are the raw projections of one dtype, with row
     strides; they pass SiLU in float32 on the way in (``activation``).  ``state``: per slot
     ``heads * vdim * dim`` float32, left as after each sequence's last token.  Returns
     ``(T, heads * vdim)`` float32.  Long portions take the chunked kernels
-    (``decay_attention_chunked``)."""
+    (``decay_attention_chunked``; ``longest``: the most tokens a sequence brings, where known)."""
     T = q.shape[0]
     ldq, ldk, ldv = _rows(q, "decay_attention q"), _rows(k, "decay_attention k"), \
         _rows(v, "decay_attention v")
@@ -271,7 +278,7 @@ def decay_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: to
                           "dtype")
     stride = _state(state, heads * vdim * dim, "decay_attention")
     out = torch.empty((T, heads * vdim), dtype=torch.float32, device=q.device)
-    if decay_attention_chunked(T, num_seqs, dim, vdim, q.dtype):
+    if decay_attention_chunked(T, num_seqs, dim, vdim, q.dtype, longest):
         max_chunks = T // DECAY_CHUNK_LEN + num_seqs        # an upper bound, known on the host
         ws = torch.empty((max_chunks, heads * vdim * dim), dtype=torch.float32, device=q.device)
         lib.call("rlis_decay_attention_chunks", out.data_ptr(), q.data_ptr(), ldq, k.data_ptr(),

@@ -358,7 +358,7 @@ class DecayAttention(Mixer):
         c = self.cols
         o = ops.decay_attention(p[:, c["q"]:c["q"] + H * d], p[:, c["k"]:c["k"] + H * d],
                                 p[:, c["v"]:c["v"] + H * dv], self.decay, S, cu, slots, n,
-                                H, d, dv)
+                                H, d, dv, longest=getattr(step, "max_new", None))
         y = ops.head_norm_gate(o, self.norm, p[:, c["g"]:c["g"] + H * dv], 1, H * dv, self.eps,
                                self.act_dtype, sigmoid_gate=True)
         return ops.pending_linear(y, self.w_o, self.act_dtype)

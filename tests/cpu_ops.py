@@ -29,7 +29,8 @@ def depth_mix_(x, delta, history, count, weights, save_input=False):
     x.copy_(sum(weights[j].float() * history[j] for j in range(count)))
 
 
-def decay_attention(q, k, v, decay, state, cu, slots, num_seqs, heads, dim, vdim, activation=True):
+def decay_attention(q, k, v, decay, state, cu, slots, num_seqs, heads, dim, vdim, activation=True,
+                    longest=None):
     T = q.shape[0]
     act = (lambda z: z / (1.0 + torch.exp(-z))) if activation else (lambda z: z)
     qq, kk = act(q.float()).reshape(T, heads, dim), act(k.float()).reshape(T, heads, dim)

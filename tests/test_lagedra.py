@@ -250,6 +250,16 @@ def test_prompts_of_hundreds_of_tokens_at_head_sizes_of_real_models(backend, dty
     steps, peak = traces.trace_mixed(reqs, live=3, seed=6)
     check_trace(runner_for(folder, backend, dtype, num_pages=-(-peak // 16), max_num_seqs=3,
                            max_positions=1024), steps, reqs, cfg, stored, dtype)
+    # a long portion beside single decoded tokens of two other requests, in one step
+    reqs = traces.random_requests(cfg["vocab"], [60, 70, 330], seed=72)
+    a, b, c = (reqs[r] for r in ("r0", "r1", "r2"))
+    cuts = [{"r0": (0, 40), "r1": (0, 50)}, {"r0": (40, 41), "r1": (50, 51), "r2": (0, 300)},
+            {"r0": (41, 60), "r1": (51, 70), "r2": (300, 330)}]
+    steps = [{"step": i, "end": [], "entries": [
+        {"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
+        for rid, (lo, hi) in cut.items()]} for i, cut in enumerate(cuts)]
+    steps[-1]["end"] = ["r0", "r1", "r2"]
+    check_trace(make(), steps, reqs, cfg, stored, dtype)
 
 
 # ------------------------------------------------------------- keys made to stand out

@@ -118,6 +118,9 @@ def test_the_chunked_form_is_chosen_by_the_steps_shape():
     assert not chosen(255, 1, 64, 64, f32)          # short steps walk token by token
     assert not chosen(2048, 40, 64, 64, f32)        # and so do steps of many short portions
     assert not chosen(2048, 1, 160, 64, f32) and not chosen(2048, 1, 64, 64, bf16)
+    # a long portion beside many decoded tokens
+    assert chosen(2048 + 200, 201, 64, 64, f32, longest=2048)
+    assert not chosen(400, 201, 64, 64, f32, longest=200)
 
 
 @pytest.mark.parametrize("T, C", [(5, 48), (3, 1000), (1, 7)])
