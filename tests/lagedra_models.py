@@ -100,7 +100,22 @@ CONFIG_D = {
         _attention(4, 2, 48, 64, 2, 300, 48, 20000.0, (2.0, 512, 8.0, 1.0), 0.14, 10.0, True, None),
     ],
 }
-CONFIGS = {"a": CONFIG_A, "b": CONFIG_B, "c": CONFIG_C, "d": CONFIG_D}
+# A width, feed-forward widths and a vocabulary that are no multiples of 8 (rows that do not
+# start on 16-byte boundaries in bfloat16), one head.  Every expert is chosen: behind a choice
+# that bfloat16 rounding can flip, the head that forgets nothing would carry the other expert's
+# output through all later rows.
+CONFIG_E = {
+    "architecture": "Lagedra", "vocab": 333, "width": 100, "max_positions": 260,
+    "norm": {"eps": 1e-5},
+    "layers": [
+        _lightning(1, 36, 52, [0.93], _moe(30, 1.0, 3, 1, 1, 3)),
+        _attention(1, 1, 28, 36, 3, 24, 14, 5000.0, (4.0, 48, 4.0, 1.0), 0.2, 12.0, True,
+                   _dense(150)),
+        _attention(3, 1, 20, 36, 2, 60, 20, 900.0, None, 0.22, 6.0, True, _moe(25, 3.0, 6, 2, 2, 6)),
+        _lightning(5, 20, 12, [0.6, 0.8, 0.9, 0.95, 1.0], _dense(70)),
+    ],
+}
+CONFIGS = {"a": CONFIG_A, "b": CONFIG_B, "c": CONFIG_C, "d": CONFIG_D, "e": CONFIG_E}
 
 
 def spec_of(config: dict):

@@ -158,7 +158,7 @@ def test_the_plain_implementation_does_not_look_ahead():
 
 
 # --------------------------------------------------------------------- the step function
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "e"])
 def test_whole_prompts_and_first_tokens(backend, dtype, name, tmp_path_factory):
     folder, cfg, stored = model_case(name, dtype, tmp_path_factory)
     reqs = traces.random_requests(cfg["vocab"], [1, 2, 3, 19, 70], seed=11)
@@ -191,7 +191,7 @@ def test_portions_of_any_size(backend, dtype, name, tmp_path_factory):
     check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
 
 
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "e"])
 def test_mixed_batches_reuse_pages_and_state_slots(backend, dtype, name, tmp_path_factory):
     """Seven unequal requests through three state slots and a pool that holds three of them:
     portions beside single tokens, requests left out of steps, slots and pages of finished
