@@ -206,6 +206,29 @@ def test_embedding_with_learned_positions_gelu_and_depth_mix(dtype):
         assert rel(history[i + 1].cpu(), kept[i + 1]) < 1e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T, W", [(1, 40), (9, 256), (70, 100)])
+def test_norm_whose_weight_is_one_number(T, W, dtype):
+    """The norm part with a weight without axes, on a stream with a delta still to be added:
+    the sum is normalised, in float32, and the stream keeps it."""
+    from rust_llm_inference_server_amd.parts.base import (BuildContext, PartSpec, ResidualStream,
+                                                          create)
+    g = torch.Generator().manual_seed(T + W)
+    weight = torch.tensor(1.7).to(dtype)
+    ctx = BuildContext(device=torch.device(DEV), act_dtype=dtype, weights={"n": weight.to(DEV)},
+                       max_positions=16)
+    norm = create("norm", PartSpec("rmsnorm", {"size": W, "eps": 1e-5, "scalar": True,
+                                               "weight_name": ""}), "n", ctx)
+    x, delta = torch.randn(T, W, generator=g) * 2.0, torch.randn(T, W, generator=g)
+    stream = ResidualStream(x.to(DEV), dtype)
+    stream.add(delta.to(DEV))
+    h = norm.forward(stream)
+    h = h if isinstance(h, torch.Tensor) else h.tensor()
+    want = plain.scalar_norm(x.double() + delta.double(), weight.double(), 1e-5)
+    assert rel(h.cpu(), want) < (1e-6 if dtype == torch.float32 else 4e-3)
+    assert rel(stream.flush().cpu(), x.double() + delta.double()) < 1e-6
+
+
 def test_rotation_tables_with_stretched_frequencies():
     """The tables of the rotation part against the plain formulas: ramps that begin at pair 0,
     that end before the last pair, that are one pair wide; the magnitude on both tables."""
