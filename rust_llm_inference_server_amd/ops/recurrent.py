@@ -236,13 +236,15 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, he
 
 # A step of at least DECAY_CHUNKED_MIN_TOKENS tokens whose sequences bring at least
 # DECAY_CHUNKED_MIN_MEAN_TOKENS each on average, or any step in which one sequence brings
-# DECAY_CHUNKED_MIN_TOKENS (a long portion beside decoded tokens), takes the chunked form of the
+# DECAY_CHUNKED_MIN_LONGEST (a portion beside decoded tokens: token by token it would take
+# 0.8 us a token, however few the others are), takes the chunked form of the
 # linear attention (chunks of DECAY_CHUNK_LEN tokens on the matrix cores, float32 products; heads
 # of at most DECAY_CHUNKED_MAX_DIM channels); every other step walks token by token.  The two
 # agree to rounding.  The rule looks at what the host knows: rows and sequences of the step and
 # its longest portion.
 DECAY_CHUNKED_MIN_TOKENS = 256
 DECAY_CHUNKED_MIN_MEAN_TOKENS = 64
+DECAY_CHUNKED_MIN_LONGEST = 64
 DECAY_CHUNKED_MAX_DIM = 128
 DECAY_CHUNK_LEN = 64
 
@@ -251,7 +253,7 @@ def decay_attention_chunked(T: int, num_seqs: int, dim: int, vdim: int, dtype: t
                             longest: Optional[int] = None) -> bool:
     if dtype != torch.float32 or max(dim, vdim) > DECAY_CHUNKED_MAX_DIM:
         return False
-    if longest is not None and longest >= DECAY_CHUNKED_MIN_TOKENS:
+    if longest is not None and longest >= DECAY_CHUNKED_MIN_LONGEST:
         return True
     return (T >= DECAY_CHUNKED_MIN_TOKENS
             and T >= DECAY_CHUNKED_MIN_MEAN_TOKENS * max(1, num_seqs))

@@ -70,6 +70,7 @@ def test_linear_attention_with_a_decay_per_head(heads, d, dv, dtype, form, monke
     steps = STEPS if form == "scan" else LONG_STEPS
     if form == "scan":
         monkeypatch.setattr(recurrent, "DECAY_CHUNKED_MIN_TOKENS", 1 << 30)
+        monkeypatch.setattr(recurrent, "DECAY_CHUNKED_MIN_LONGEST", 1 << 30)
     elif form == "chunks":
         if dtype != torch.float32 or max(d, dv) > 128:
             pytest.skip("the chunked form takes float32 rows and heads of up to 128 channels")
@@ -120,7 +121,7 @@ def test_the_chunked_form_is_chosen_by_the_steps_shape():
     assert not chosen(2048, 1, 160, 64, f32) and not chosen(2048, 1, 64, 64, bf16)
     # a long portion beside many decoded tokens
     assert chosen(2048 + 200, 201, 64, 64, f32, longest=2048)
-    assert not chosen(400, 201, 64, 64, f32, longest=200)
+    assert chosen(90, 21, 64, 64, f32, longest=70) and not chosen(400, 201, 64, 64, f32, longest=50)
 
 
 @pytest.mark.parametrize("T, C", [(5, 48), (3, 1000), (1, 7)])
