@@ -252,7 +252,6 @@ def test_prompts_of_hundreds_of_tokens_at_head_sizes_of_real_models(backend, dty
                            max_positions=1024), steps, reqs, cfg, stored, dtype)
     # a long portion beside single decoded tokens of two other requests, in one step
     reqs = traces.random_requests(cfg["vocab"], [60, 70, 330], seed=72)
-    a, b, c = (reqs[r] for r in ("r0", "r1", "r2"))
     cuts = [{"r0": (0, 40), "r1": (0, 50)}, {"r0": (40, 41), "r1": (50, 51), "r2": (0, 300)},
             {"r0": (41, 60), "r1": (51, 70), "r2": (300, 330)}]
     steps = [{"step": i, "end": [], "entries": [

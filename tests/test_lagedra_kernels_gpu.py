@@ -91,7 +91,7 @@ def test_linear_attention_with_a_decay_per_head(heads, d, dv, dtype, form, monke
                                       x["v"].reshape(-1, heads, dv), decay, Sx))
         S.append(Sx)
     at_seq = [0, 0, 0]
-    tol = 2e-5 if dtype == torch.float32 else 2e-5       # the inputs are rounded, not the sums
+    tol = 2e-5             # in either dtype: the inputs are rounded, not the sums
     for lengths in steps:
         cu, slots, _ = _meta(lengths, SLOTS)
         rows = {n: torch.cat([data[i][n][at_seq[i]:at_seq[i] + lengths[i]] for i in range(3)])
