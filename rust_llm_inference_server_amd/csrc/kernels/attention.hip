@@ -34,7 +34,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, int nh, int nkv, int d, int page_size, float scale,
     int window, const float* __restrict__ slopes, const float* __restrict__ head_scales,
-    float softcap) {
+    float softcap, const float* __restrict__ sinks, int keep_first) {
   extern __shared__ float smem[];
   float* q_s = smem;                          // d
   float* p_s = smem + d;                      // 64
@@ -54,9 +54,14 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
   float acc[DPL];
 #pragma unroll
   for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
-  for (int k0 = lo; k0 <= pos; k0 += 64) {
+  // two runs of keys: the sequence's first keys that stay visible in front of the window
+  // (none without a window), then the window up to the query itself
+  const int kept = min(keep_first, lo);
+  for (int run = kept > 0 ? 0 : 1; run < 2; ++run) {
+  const int run_end = run == 0 ? kept : pos + 1;
+  for (int k0 = run == 0 ? 0 : lo; k0 < run_end; k0 += 64) {
     const int kpos = k0 + lane;
-    const bool valid = kpos <= pos;
+    const bool valid = kpos < run_end;
     float s = -INFINITY;
     long long vbase = 0;
     if (valid) {
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     p_s[lane] = p;
     vbase_s[lane] = vbase;
     __syncthreads();
-    const int n = min(64, pos - k0 + 1);
+    const int n = min(64, run_end - k0);
 #pragma unroll
     for (int i = 0; i < DPL; ++i) {
       const int j = lane + 64 * i;
@@ -89,6 +94,16 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(
     }
     __syncthreads();
     m = m_new;
+  }
+  }
+  if (sinks) {
+    // the sink counts once in the denominator: e^sink beside the keys' e^score
+    const float sink = sinks[h];
+    const float m_new = fmaxf(m, sink);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(sink - m_new);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) acc[i] *= corr;
   }
   const float inv_l = 1.0f / l;
 #pragma unroll
@@ -103,8 +118,10 @@ RLIS_API int rlis_attn_generic(const void* q, int dtype, long long q_stride, voi
                                const int* block_tables, int max_pages, const int* seq_of_token,
                                const int* positions, int T, int nh, int nkv, int d, int page_size,
                                float scale, int window, const float* slopes,
-                               const float* head_scales, float softcap, hipStream_t stream) {
+                               const float* head_scales, float softcap, const float* sinks,
+                               int keep_first, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_generic: bad sizes");
+  RLIS_REQUIRE(keep_first >= 0, "attn_generic: bad count of kept first keys");
   RLIS_REQUIRE(nh % nkv == 0, "attn_generic: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
   RLIS_REQUIRE(d <= 512 && d % 2 == 0, "attn_generic: head_dim %d must be even and at most 512", d);
@@ -117,7 +134,7 @@ RLIS_API int rlis_attn_generic(const void* q, int dtype, long long q_stride, voi
   attn_generic_kernel<TX, DPL><<<grid, 64, smem, stream>>>(                                    \
       (const TX*)q, q_stride, (TX*)out, out_stride, (const TX*)k_pages, (const TX*)v_pages,    \
       block_tables, max_pages, seq_of_token, positions, nh, nkv, d, page_size, scale, window,  \
-      slopes, head_scales, softcap)
+      slopes, head_scales, softcap, sinks, keep_first)
 #define BY_DPL(TX)                         \
   do {                                     \
     if (dpl <= 1) LAUNCH(TX, 1);           \
@@ -173,7 +190,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int* __restrict__ ctx_lens, const int* __restrict__ token_rows, int nh, int nkv, int d,
     int page_size, float scale, int window, int splits, int chunks_per_kv, int part_keys,
     int max_parts, const float* __restrict__ slopes, const float* __restrict__ head_scales,
-    float softcap) {
+    float softcap, const float* __restrict__ sinks, int keep_first) {
   extern __shared__ float smem[];
   float* q_s = smem;                     // G * d
   float* p_s = q_s + G * d;              // 4 waves * G * 64
@@ -220,12 +237,17 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   // a multiple of VN and the page size is one.
   const bool vec_ok = (kbeg % VN == 0) && (page_size % VN == 0);
 
+  // The sequence's first keys that stay visible in front of the window go to its first
+  // partition, ahead of that partition's own keys.
+  const int kept = split == 0 ? min(keep_first, lo) : 0;
+  for (int run = kept > 0 ? 0 : 1; run < 2; ++run) {
+  const int rbeg = run == 0 ? 0 : kbeg, rend = run == 0 ? kept : kend;
   // Every wave runs the same number of rounds so that the block-wide barriers match.
-  const int rounds = kend > kbeg ? (kend - kbeg + 255) / 256 : 0;
+  const int rounds = rend > rbeg ? (rend - rbeg + 255) / 256 : 0;
   for (int it = 0; it < rounds; ++it) {
-    const int k0 = kbeg + it * 256 + wave * 64;
+    const int k0 = rbeg + it * 256 + wave * 64;
     const int kpos = k0 + lane;
-    const bool valid = kpos < kend;
+    const bool valid = kpos < rend;
     float s[G];
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) s[hh] = 0.f;
@@ -261,7 +283,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
     my_vbase[lane] = vbase;
     __syncthreads();
-    const int n = max(0, min(64, kend - k0));
+    const int n = max(0, min(64, rend - k0));
+    const bool vec_run = run == 0 ? (page_size % VN == 0) : vec_ok;
 #pragma unroll
     for (int i = 0; i < DPL; ++i) {
       const int j = lane + 64 * i;
@@ -270,7 +293,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       for (int hh = 0; hh < G; ++hh) a[hh] = acc[hh][i] * corr[hh];
       if (j < d) {
         int kk = 0;
-        if (vec_ok) {
+        if (vec_run) {
           for (; kk + VN <= n; kk += VN) {
             float v[VN];
             Vec16<TX>::load(v_pages + my_vbase[kk] + (long long)j * page_size, v);
@@ -290,6 +313,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       for (int hh = 0; hh < G; ++hh) acc[hh][i] = a[hh];
     }
     __syncthreads();
+  }
   }
 
   // Merge the four waves in order.
@@ -322,6 +346,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     }
     const int h = h0 + hh;
     if (splits == 1) {
+      if (sinks) {
+        // (no key at all cannot be: a query sees itself)
+        const float sink = sinks[h];
+        const float top = fmaxf(big, sink);
+        const float e = expf(big - top);
+        a *= e;
+        lsum = lsum * e + expf(sink - top);
+      }
       st(out + (long long)row * out_stride + h * d + j, a / lsum);
     } else {
       const long long idx = ((long long)seq * nh + h) * splits + split;
@@ -351,7 +383,8 @@ __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
                                    const float* __restrict__ part_acc,
                                    const int* __restrict__ token_rows, int nh, int d, int stride,
                                    const int* __restrict__ seq_of_row,
-                                   const int* __restrict__ seq_parts, int row0) {
+                                   const int* __restrict__ seq_parts, int row0,
+                                   const float* __restrict__ sinks) {
   extern __shared__ float reduce_w[];            // stride weights, then 8 floats of scratch
   float* scratch = reduce_w + stride;
   const int h = blockIdx.x, seq = blockIdx.y;
@@ -375,6 +408,8 @@ __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
   if (lane == 0) scratch[wave] = big;
   __syncthreads();
   for (int w = 0; w < nwaves; ++w) big = fmaxf(big, scratch[w]);
+  // a sink joins as one more partition that holds e^sink in its denominator and no values
+  if (sinks) big = fmaxf(big, sinks[h]);
   for (int s = threadIdx.x; s < splits; s += blockDim.x) {
     const float ls = part_ml[(base + s) * 2 + 1];
     reduce_w[s] = ls > 0.f ? expf(part_ml[(base + s) * 2] - big) : 0.f;
@@ -385,6 +420,7 @@ __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
     const float e = reduce_w[s];
     if (e > 0.f) lsum += part_ml[(base + s) * 2 + 1] * e;
   }
+  if (sinks) lsum += expf(sinks[h] - big);
   for (int j = threadIdx.x; j < d; j += blockDim.x) {
     float a = 0.f;
     const float* acc = part_acc + base * d + j;
@@ -411,11 +447,12 @@ __global__ void attn_reduce_kernel(TX* __restrict__ out, long long out_stride,
 // matrix-core decode kernel, which lives in another unit).
 int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* part_ml,
                                  const float* part_acc, int S, int nh, int d, int splits,
-                                 hipStream_t stream) {
+                                 const float* sinks, hipStream_t stream) {
   dim3 grid(nh, S);
   const int threads = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
   attn_reduce_kernel<bf16_t><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
-      (bf16_t*)out, out_stride, part_ml, part_acc, nullptr, nh, d, splits, nullptr, nullptr, 0);
+      (bf16_t*)out, out_stride, part_ml, part_acc, nullptr, nh, d, splits, nullptr, nullptr, 0,
+      sinks);
   RLIS_LAUNCH_CHECK("attn_reduce");
   return 0;
 }
@@ -431,7 +468,7 @@ __global__ __launch_bounds__(256) void attn_reduce_rows_kernel(
     bf16_t* __restrict__ out, long long out_stride, const float* __restrict__ part_ml,
     const float* __restrict__ part_acc, int nh, int d, int stride,
     const int* __restrict__ seq_of_row, const int* __restrict__ seq_parts, int row0,
-    long long pairs) {
+    long long pairs, const float* __restrict__ sinks) {
   const long long pair = (long long)blockIdx.x * 4 + threadIdx.x / kWave;
   if (pair >= pairs) return;
   const int lane = threadIdx.x % kWave;
@@ -453,8 +490,9 @@ __global__ __launch_bounds__(256) void attn_reduce_rows_kernel(
     if (lv[s] > 0.f) big = fmaxf(big, mv[s]);
   for (int s = kRowRuns; s < splits; ++s)
     if (part_ml[(base + s) * 2 + 1] > 0.f) big = fmaxf(big, part_ml[(base + s) * 2]);
+  if (sinks) big = fmaxf(big, sinks[h]);
   float ev[kRowRuns];
-  float lsum = 0.f;
+  float lsum = sinks ? expf(sinks[h] - big) : 0.f;
 #pragma unroll
   for (int s = 0; s < kRowRuns; ++s) {
     ev[s] = lv[s] > 0.f ? expf(mv[s] - big) : 0.f;
@@ -490,7 +528,7 @@ __global__ __launch_bounds__(256) void attn_reduce_rows_kernel(
 RLIS_API int rlis_attn_reduce_rows(void* out, long long out_stride, const float* part_ml,
                                    const float* part_acc, const int* seq_of_token,
                                    const int* seq_runs, int row0, int rows, int nh, int d,
-                                   int stride, hipStream_t stream) {
+                                   int stride, const float* sinks, hipStream_t stream) {
   RLIS_REQUIRE(rows >= 0 && row0 >= 0 && nh > 0 && d > 0 && stride >= 1 && stride <= 64,
                "attn_reduce_rows: bad sizes");
   RLIS_REQUIRE(part_ml && part_acc && seq_of_token && seq_runs,
@@ -501,7 +539,7 @@ RLIS_API int rlis_attn_reduce_rows(void* out, long long out_stride, const float*
   if (pairs > 0)
     attn_reduce_rows_kernel<<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(
         (bf16_t*)out, out_stride, part_ml, part_acc, nh, d, stride, seq_of_token, seq_runs, row0,
-        pairs);
+        pairs, sinks);
   RLIS_LAUNCH_CHECK("attn_reduce_rows");
   return 0;
 }
@@ -513,7 +551,7 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
                          const int* ctx_lens, const int* token_rows, int S, int nh, int nkv, int d,
                          int page_size, float scale, int window, int splits, int part_keys,
                          int max_parts, const float* slopes, const float* head_scales,
-                         float softcap, hipStream_t stream) {
+                         float softcap, const float* sinks, int keep_first, hipStream_t stream) {
   const int g = nh / nkv;
   const int chunks = ceil_div(g, G);
   dim3 grid(nkv * chunks, S, splits);
@@ -525,7 +563,8 @@ static int launch_decode(const void* q, long long q_stride, void* out, long long
   attn_decode_kernel<TX, G, DPL><<<grid, 256, smem, stream>>>(                                 \
       (const TX*)q, q_stride, (TX*)out, out_stride, part_ml, part_acc, (const TX*)k_pages,     \
       (const TX*)v_pages, block_tables, max_pages, ctx_lens, token_rows, nh, nkv, d, page_size, \
-      scale, window, splits, chunks, part_keys, max_parts, slopes, head_scales, softcap)
+      scale, window, splits, chunks, part_keys, max_parts, slopes, head_scales, softcap,       \
+      sinks, keep_first)
   if (dpl <= 1) LAUNCH(1);
   else if (dpl <= 2) LAUNCH(2);
   else LAUNCH(4);
@@ -544,7 +583,8 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
                               int max_pages, const int* ctx_lens, const int* token_rows, int S,
                               int nh, int nkv, int d, int page_size, float scale, int window,
                               int splits, int part_keys, int max_parts, const float* slopes,
-                              const float* head_scales, float softcap, hipStream_t stream) {
+                              const float* head_scales, float softcap, const float* sinks,
+                              int keep_first, hipStream_t stream) {
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode: bad sizes");
   RLIS_REQUIRE(part_keys >= 64 && part_keys % 64 == 0 && max_parts >= 1 && splits <= max_parts,
                "attn_decode: partitions of %d keys (a multiple of 64), %d deep of at most %d",
@@ -564,22 +604,22 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
       rc = launch_decode<TX, 1>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, head_scales, softcap, stream);               \
+                                slopes, head_scales, softcap, sinks, keep_first, stream); \
     else if (g == 2)                                                                             \
       rc = launch_decode<TX, 2>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, head_scales, softcap, stream);               \
+                                slopes, head_scales, softcap, sinks, keep_first, stream); \
     else if (g <= 4)                                                                             \
       rc = launch_decode<TX, 4>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, head_scales, softcap, stream);               \
+                                slopes, head_scales, softcap, sinks, keep_first, stream); \
     else                                                                                         \
       rc = launch_decode<TX, 8>(q, q_stride, out, out_stride, part_ml, part_acc, k_pages,        \
                                 v_pages, block_tables, max_pages, ctx_lens, token_rows, S, nh,   \
                                 nkv, d, page_size, scale, window, splits, part_keys, max_parts,       \
-                                slopes, head_scales, softcap, stream);               \
+                                slopes, head_scales, softcap, sinks, keep_first, stream); \
   } while (0)
   if (dtype == RLIS_F32) BY_G(float);
   else if (dtype == RLIS_BF16) BY_G(bf16_t);
@@ -593,11 +633,11 @@ RLIS_API int rlis_attn_decode(const void* q, int dtype, long long q_stride, void
     if (dtype == RLIS_F32)
       attn_reduce_kernel<float><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
           (float*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits, nullptr, nullptr,
-          0);
+          0, sinks);
     else
       attn_reduce_kernel<bf16_t><<<grid, threads, (splits + 8) * sizeof(float), stream>>>(
           (bf16_t*)out, out_stride, part_ml, part_acc, token_rows, nh, d, splits, nullptr, nullptr,
-          0);
+          0, sinks);
     RLIS_LAUNCH_CHECK("attn_reduce");
   }
   return 0;

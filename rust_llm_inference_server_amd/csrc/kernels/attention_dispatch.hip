@@ -60,7 +60,7 @@ static int unit_result(const char* name, int rc, int d) {
 
 int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* part_ml,
                                  const float* part_acc, int S, int nh, int d, int splits,
-                                 hipStream_t stream);
+                                 const float* sinks, hipStream_t stream);
 
 // unit_map lists num_units quadruples (sequence, first new-token index of a tile, run, runs of
 // the sequence): the keys of a tile of a sequence with more than one run are cut into that
@@ -216,6 +216,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0 && !inside)
-    return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, stream);
+    return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, nullptr,
+                                        stream);
   return 0;
 }

@@ -937,7 +937,8 @@ RLIS_API int rlis_rope_kv_write(void* qkv, int dtype, long long row_stride, int 
                                 const float* sin_t, const int* positions, const int* slots,
                                 void* k_pages, void* v_pages, int page_size, int write_kv,
                                 int interleaved, int rotate_q, hipStream_t stream) {
-  RLIS_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && d > 0, "rope_kv_write: bad sizes");
+  RLIS_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && (nkv > 0 || !write_kv) && d > 0,
+               "rope_kv_write: bad sizes");
   RLIS_REQUIRE(rot_dim >= 0 && rot_dim <= d && rot_dim % 2 == 0,
                "rope_kv_write: rot_dim %d must be even and at most head_dim %d", rot_dim, d);
   RLIS_REQUIRE(!write_kv || (page_size > 0 && k_pages && v_pages && slots),

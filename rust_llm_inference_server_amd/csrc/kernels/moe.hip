@@ -99,6 +99,13 @@ RLIS_API int rlis_moe_router_logits(const float* resid, const void* ln_w, const 
 
 // What a unit makes of its gate and up products: silu(g) * u, or with limit > 0 the bounded
 // form g' * sigmoid(alpha * g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).
+// With alpha < 0 the unit is not gated at all: the two products are two halves of one
+// projection's columns and each goes through the squared ReLU by itself (see plain_unit).
+__device__ __forceinline__ float plain_unit(float z) {
+  const float r = fmaxf(z, 0.f);
+  return r * r;
+}
+
 __device__ __forceinline__ float gated_unit(float g, float u, float limit, float alpha) {
   if (limit > 0.f) {
     g = fminf(g, limit);
@@ -124,7 +131,7 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
 __global__ __launch_bounds__(64) void moe_route_kernel(
     const float* __restrict__ z, long long ldz, const float* __restrict__ correction, int E,
     int G, int keep, int top, float scale, int* __restrict__ chosen, float* __restrict__ weights,
-    int softmax_scores, int group_max, int renormalise) {
+    int softmax_scores, int group_max, int renormalise, const float* __restrict__ bias) {
   extern __shared__ float sm[];
   float* choice = sm;            // E
   float* gscore = sm + E;        // G
@@ -133,14 +140,16 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
   const int per = E / G;
   float zmax = -INFINITY, zsum = 1.f;
   if (softmax_scores) {
-    for (int e = lane; e < E; e += 64) zmax = fmaxf(zmax, z[(long long)t * ldz + e]);
+    for (int e = lane; e < E; e += 64)
+      zmax = fmaxf(zmax, z[(long long)t * ldz + e] + (bias ? bias[e] : 0.f));
     zmax = wave_max(zmax);
     float part = 0.f;
-    for (int e = lane; e < E; e += 64) part += expf(z[(long long)t * ldz + e] - zmax);
+    for (int e = lane; e < E; e += 64)
+      part += expf(z[(long long)t * ldz + e] + (bias ? bias[e] : 0.f) - zmax);
     zsum = wave_sum(part);
   }
   for (int e = lane; e < E; e += 64) {
-    const float zv = z[(long long)t * ldz + e];
+    const float zv = z[(long long)t * ldz + e] + (bias ? bias[e] : 0.f);
     const float s = softmax_scores ? expf(zv - zmax) / zsum : 1.0f / (1.0f + expf(-zv));
     score[e] = s;
     choice[e] = s + (correction ? correction[e] : 0.f);
@@ -197,7 +206,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(
 RLIS_API int rlis_moe_route(const float* z, long long ldz, const float* correction, int T, int E,
                             int G, int keep, int top, float scale, int* chosen, float* weights,
                             int softmax_scores, int group_max, int renormalise,
-                            hipStream_t stream) {
+                            const float* bias, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && E > 0 && G > 0 && E % G == 0 && keep >= 1 && keep <= G && top >= 1,
                "moe_route: bad sizes E=%d groups=%d keep=%d top=%d", E, G, keep, top);
   RLIS_REQUIRE(top <= keep * (E / G), "moe_route: %d experts asked of %d allowed", top,
@@ -206,7 +215,7 @@ RLIS_API int rlis_moe_route(const float* z, long long ldz, const float* correcti
   if (T == 0) return 0;
   moe_route_kernel<<<T, 64, (size_t)(2 * E + G) * 4, stream>>>(
       z, ldz, correction, E, G, keep, top, scale, chosen, weights, softmax_scores, group_max,
-      renormalise);
+      renormalise, bias);
   RLIS_LAUNCH_CHECK("moe_route");
   return 0;
 }
@@ -290,7 +299,14 @@ __global__ __launch_bounds__(64 * WAVES) void moe_gate_up_kernel(
     for (int i = 0; i < 4; ++i) {
       const int row = row0 + (lane / 16) * 4 + i;
       const float g = acc[b][i], u = acc[b + 2][i];
-      if (f < F) st(hidden + (long long)row * F + f, gated_unit(g, u, limit, alpha));
+      if (f < F) {
+        if (alpha < 0.f) {
+          st(hidden + (long long)row * 2 * F + f, plain_unit(g));
+          st(hidden + (long long)row * 2 * F + F + f, plain_unit(u));
+        } else {
+          st(hidden + (long long)row * F + f, gated_unit(g, u, limit, alpha));
+        }
+      }
     }
   }
 }
@@ -368,7 +384,14 @@ __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(
       for (int i = 0; i < 4; ++i) {
         const int row = row0 + a * 16 + (lane / 16) * 4 + i;
         const float g = acc[a][b][i], u = acc[a][b + 2][i];
-        if (f < F) st(hidden + (long long)row * F + f, gated_unit(g, u, limit, alpha));
+        if (f < F) {
+          if (alpha < 0.f) {
+            st(hidden + (long long)row * 2 * F + f, plain_unit(g));
+            st(hidden + (long long)row * 2 * F + F + f, plain_unit(u));
+          } else {
+            st(hidden + (long long)row * F + f, gated_unit(g, u, limit, alpha));
+          }
+        }
       }
     }
 }
@@ -519,7 +542,14 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(
       if (GATE_UP) {
         const int f = n0 + wn * 32 + lane % 32;
         const float g = acc[i][0][r], u = acc[i][1][r];
-        if (f < N) hidden[(long long)row * N + f] = f32_to_bf16(gated_unit(g, u, limit, alpha));
+        if (f < N) {
+          if (alpha < 0.f) {
+            hidden[(long long)row * 2 * N + f] = f32_to_bf16(plain_unit(g));
+            hidden[(long long)row * 2 * N + N + f] = f32_to_bf16(plain_unit(u));
+          } else {
+            hidden[(long long)row * N + f] = f32_to_bf16(gated_unit(g, u, limit, alpha));
+          }
+        }
       } else {
         const int pair = sorted[row];
         if (pair < 0) continue;
@@ -543,18 +573,21 @@ RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const voi
                "moe_experts: bad sizes");
   RLIS_REQUIRE(ldx >= K, "moe_experts: row stride shorter than a row");
   if (max_tiles == 0) return 0;
+  // plain units (alpha < 0): the up projection's 2 F columns are the hidden row, F "gate"
+  // columns in front of F "up" columns, and the down product runs over all of them
+  const int FD = alpha < 0.f ? 2 * F : F;
   if (tile_rows == 128) {
     RLIS_REQUIRE(dtype == RLIS_BF16 && mma_rows_aligned<bf16_t>(x, ldx, 0, K) &&
                      mma_rows_aligned<bf16_t>(w_gu, K, 0, K) &&
-                     mma_rows_aligned<bf16_t>(hidden, F, 0, F) &&
-                     mma_rows_aligned<bf16_t>(w_d, F, 0, F),
+                     mma_rows_aligned<bf16_t>(hidden, FD, 0, FD) &&
+                     mma_rows_aligned<bf16_t>(w_d, FD, 0, FD),
                  "moe_experts: tiles of 128 rows take bfloat16 rows on 16-byte boundaries");
     RLIS_REQUIRE(ceil_div(F, 64) <= 65535 && ceil_div(K, 128) <= 65535, "moe_experts: too wide");
     moe_tiles128_kernel<true><<<dim3(max_tiles, ceil_div(F, 64)), 256, 0, stream>>>(
         (const bf16_t*)x, ldx, (const bf16_t*)w_gu, sorted, tile_expert, weights, top, F, K,
         (bf16_t*)hidden, nullptr, limit, alpha);
     moe_tiles128_kernel<false><<<dim3(max_tiles, ceil_div(K, 128)), 256, 0, stream>>>(
-        (const bf16_t*)hidden, F, (const bf16_t*)w_d, sorted, tile_expert, weights, top, K, F,
+        (const bf16_t*)hidden, FD, (const bf16_t*)w_d, sorted, tile_expert, weights, top, K, FD,
         nullptr, y, 0.f, 0.f);
     RLIS_LAUNCH_CHECK("moe_experts");
     return 0;
@@ -568,19 +601,19 @@ RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const voi
           (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden, limit, \
           alpha);                                                                              \
       moe_down_rows_kernel<T, AL2><<<dim3(max_tiles, ceil_div(K, 256)), 256, 0, stream>>>(     \
-          (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);             \
+          (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, FD, y);            \
     } else {                                                                                   \
       moe_gate_up_kernel<T, WAVES, AL1><<<g1, 64 * WAVES, 0, stream>>>(                        \
           (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden, limit, \
           alpha);                                                                              \
       moe_down_kernel<T, WAVES, AL2><<<g2, 64 * WAVES, 0, stream>>>(                           \
-          (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);             \
+          (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, FD, y);            \
     }                                                                                          \
   } while (0)
 #define BY_ALIGN(T, WAVES)                                                                    \
   do {                                                                                        \
     const bool a1 = mma_rows_aligned<T>(x, ldx, 0, K) && mma_rows_aligned<T>(w_gu, K, 0, K);  \
-    const bool a2 = mma_rows_aligned<T>(hidden, F, 0, F) && mma_rows_aligned<T>(w_d, F, 0, F); \
+    const bool a2 = mma_rows_aligned<T>(hidden, FD, 0, FD) && mma_rows_aligned<T>(w_d, FD, 0, FD); \
     if (a1 && a2) LAUNCH(T, WAVES, true, true);                                               \
     else if (a1) LAUNCH(T, WAVES, true, false);                                               \
     else if (a2) LAUNCH(T, WAVES, false, true);                                               \

@@ -205,6 +205,143 @@ def gelu_tanh(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    """``0.5 x (1 + erf(x / sqrt 2))``, float32 arithmetic."""
+    _check(x, "gelu_erf")
+    if not x.is_contiguous():
+        raise KernelError("gelu_erf: tensor must be contiguous")
+    out = torch.empty_like(x)
+    lib.call("rlis_gelu_erf", out.data_ptr(), x.data_ptr(), _dt(x), x.numel(), lib.stream_ptr())
+    return out
+
+
+def lanes_step(lanes: torch.Tensor, count: int, update: Optional[tuple] = None,
+               read: Optional[torch.Tensor] = None, norm_weight: Optional[torch.Tensor] = None,
+               eps: float = 0.0, out_dtype: Optional[torch.dtype] = None,
+               rows: Optional[torch.Tensor] = None, round_parts: bool = False,
+               want: bool = True):
+    """One step over ``count`` residual streams kept side by side.
+
+    ``lanes`` is ``(count, T, H)`` float32, or ``(T, H)`` float32 when all streams still equal
+    one tensor.  ``update = (y, mix, back)``: the streams become
+    ``lanes'[t] = sum_s mix[s, t] lanes[s] + back[t] y`` (``mix (count, count)`` and
+    ``back (count)`` float32; ``y (T, H)`` in float32 or bfloat16, or a stack ``(P, T, H)`` of
+    float32 partial sums that are added in order and with ``round_parts`` rounded to bfloat16
+    first).  ``want``: the read-out ``u = sum_s read[s] lanes'[s]`` (``read`` None: the plain
+    sum) comes back, through ``u / sqrt(mean(u^2) + eps) * norm_weight`` when a weight is given,
+    in ``out_dtype`` (float32 without).  With ``rows`` (int32) only those tokens are read out,
+    and the streams stay as they are.  Returns ``(lanes', out)``; every sum is float32 and runs
+    over the streams in order."""
+    _check(lanes, "lanes", torch.float32)
+    if not lanes.is_contiguous() or lanes.dim() not in (2, 3):
+        raise KernelError("lanes_step: the streams must be contiguous (S, T, H) or (T, H)")
+    S = int(count)
+    shared = lanes.dim() == 2
+    if not shared and lanes.shape[0] != S:
+        raise KernelError(f"lanes_step: {lanes.shape[0]} streams, expected {S}")
+    T, H = lanes.shape[-2:]
+    stride = 0 if shared else T * H
+    y_ptr = mix_ptr = back_ptr = None
+    y_dt, parts, part_stride, dst = 0, 1, 0, lanes
+    store = 0
+    if update is not None:
+        y, mix, back = update
+        parts = _delta_parts(lanes[0] if not shared else lanes, y, "lanes_step")
+        for t, n, what in ((mix, S * S, "mix"), (back, S, "back")):
+            _check(t, f"lanes_step {what}", torch.float32)
+            if t.numel() != n or not t.is_contiguous():
+                raise KernelError(f"lanes_step: {what} has {t.numel()} entries, expected {n}")
+        y_ptr, y_dt, mix_ptr, back_ptr = y.data_ptr(), _dt(y), mix.data_ptr(), back.data_ptr()
+        part_stride = T * H
+        if rows is None:
+            store = 1
+            if shared:
+                dst = torch.empty((S, T, H), dtype=torch.float32, device=lanes.device)
+    read_ptr = None
+    if read is not None:
+        _check(read, "lanes_step read", torch.float32)
+        if read.numel() != S or not read.is_contiguous():
+            raise KernelError(f"lanes_step: {read.numel()} read weights for {S} streams")
+        read_ptr = read.data_ptr()
+    out = None
+    w_ptr, w_dt = None, 0
+    if want:
+        if norm_weight is not None:
+            _check(norm_weight, "norm weight", ndim=1)
+            if norm_weight.numel() != H or not norm_weight.is_contiguous():
+                raise KernelError(f"lanes_step: norm weight has {norm_weight.numel()} entries, "
+                                  f"rows have {H}")
+            w_ptr, w_dt = norm_weight.data_ptr(), _dt(norm_weight)
+        R = T if rows is None else rows.numel()
+        out = torch.empty((R, H), dtype=out_dtype or torch.float32, device=lanes.device)
+    elif rows is not None:
+        raise KernelError("lanes_step: picked rows are for reading out")
+    R = T if rows is None else rows.numel()
+    lib.call("rlis_lanes_step", lanes.data_ptr(), stride, dst.data_ptr(),
+             T * H, y_ptr, y_dt, parts, part_stride,
+             int(bool(round_parts) and parts >= 1 and update is not None and update[0].dim() == 3),
+             mix_ptr, back_ptr, read_ptr, w_ptr, w_dt, float(eps),
+             None if out is None else out.data_ptr(), 0 if out is None else _DT[out.dtype],
+             None if rows is None else _i32(rows, "rows"), R, H, S, store, lib.stream_ptr())
+    return (dst if store else lanes), out
+
+
+def head_prepare_(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                  real_dim: int, bias: Optional[torch.Tensor] = None,
+                  q_weight: Optional[torch.Tensor] = None,
+                  k_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                  positions: Optional[torch.Tensor] = None, temp_coef: float = 0.0,
+                  temp_every: int = 0) -> torch.Tensor:
+    """In place on the rows of a fused projection ``(T, >= (nh + 2 nkv) head_dim)`` (``nkv`` 0:
+    queries only): ``bias`` (float32, one per column of the heads) is added; every query and
+    key head is divided by the root mean square of its first ``real_dim`` numbers (eps inside
+    the root) and multiplied by ``q_weight`` / ``k_weight`` (float32 ``(real_dim)``, shared by
+    the heads; None: no norm); with ``temp_every`` > 0 the queries of a token at position p are
+    multiplied by ``1 + temp_coef ln(floor((p + 1) / temp_every) + 1)``.  Float32 arithmetic,
+    one rounding."""
+    stride = _rows_contig(qkv, "qkv")
+    T = qkv.shape[0]
+    nh, nkv, D = int(num_heads), int(num_kv_heads), int(head_dim)
+    cols = (nh + 2 * nkv) * D
+    if qkv.shape[1] < cols:
+        raise KernelError(f"head_prepare: rows of {qkv.shape[1]} hold no {cols} columns of heads")
+    if bias is not None:
+        _check(bias, "head_prepare bias", torch.float32, 1)
+        if bias.numel() != cols or not bias.is_contiguous():
+            raise KernelError(f"head_prepare: {bias.numel()} biases for {cols} columns")
+    for w, what in ((q_weight, "query"), (k_weight, "key")):
+        if w is not None:
+            _check(w, f"head_prepare {what} weight", torch.float32, 1)
+            if w.numel() != real_dim or not w.is_contiguous():
+                raise KernelError(f"head_prepare: the {what} norm's weight has {w.numel()} "
+                                  f"entries, a head {real_dim}")
+    pos_ptr = None
+    if temp_every > 0:
+        if positions is None:
+            raise KernelError("head_prepare: the queries' factor needs the tokens' positions")
+        pos_ptr = _i32(positions, "positions", T)
+    lib.call("rlis_head_prepare", qkv.data_ptr(), _dt(qkv), stride, T, nh, nkv, D, int(real_dim),
+             None if bias is None else bias.data_ptr(),
+             None if q_weight is None else q_weight.data_ptr(),
+             None if k_weight is None else k_weight.data_ptr(), float(eps), pos_ptr,
+             float(temp_coef), int(temp_every), lib.stream_ptr())
+    return qkv
+
+
+def head_gate_(x: torch.Tensor, gate: torch.Tensor, num_heads: int, head_dim: int
+               ) -> torch.Tensor:
+    """``x (T, nh * d)``: head h of row t times ``sigmoid(gate[t, h])``, in place (``gate``
+    ``(T, >= nh)`` of x's dtype, rows contiguous; float32 arithmetic, one rounding)."""
+    xs, gs = _rows_contig(x, "head_gate x"), _rows_contig(gate, "head_gate gate")
+    T = x.shape[0]
+    if x.shape[1] != num_heads * head_dim or gate.shape[0] != T or gate.shape[1] < num_heads \
+            or gate.dtype != x.dtype:
+        raise KernelError("head_gate: x must be (T, nh * d) and gate (T, >= nh) of one dtype")
+    lib.call("rlis_head_gate", x.data_ptr(), _dt(x), xs, gate.data_ptr(), gs, T, int(num_heads),
+             int(head_dim), lib.stream_ptr())
+    return x
+
+
 def depth_mix_(x: torch.Tensor, delta: torch.Tensor, history: torch.Tensor, count: int,
                weights: torch.Tensor, save_input: bool = False) -> None:
     """``history (slots, T, W)`` float32 holds the embedding output and every layer's result so
@@ -840,28 +977,31 @@ def _prefill_mfma_ok(qkv: torch.Tensor, d: int, page_size: int) -> bool:
 # Whether scores with a scale per head or a cap take the matrix-core kernels (False: the
 # vector-unit kernels, for tests that hold the two against each other).
 SHAPED_SCORES_MATRIX = True
+# Whether a sink in the softmax or kept first keys send a batch to the vector-unit kernels.
+PLAIN_EXTRAS = True
 
 
 def attention_planner(num_heads: int, num_kv_heads: int, head_dim: int,
                       dtype: torch.dtype, biased: bool = False,
-                      shaped: bool = False) -> AttentionPlanner:
+                      shaped: bool = False, plain: bool = False) -> AttentionPlanner:
     """The planner a mixer that calls ``paged_attention`` / ``rope_attention`` names as its
     ``step_planner()``; ``biased``: it will pass ``bias_slopes`` (the matrix-core kernels take
     them too, so the plan is the same); ``shaped``: it will pass ``head_scales`` or a
     ``softcap``."""
     return AttentionPlanner(num_heads, num_kv_heads, head_dim,
-                            matrix=dtype == torch.bfloat16
+                            matrix=dtype == torch.bfloat16 and not (plain and PLAIN_EXTRAS)
                             and (not shaped or SHAPED_SCORES_MATRIX),
                             singles_apart=SPLIT_MIXED_ATTENTION and DECODE_ATTENTION != "vector")
 
 
 def _attention_kernel(qkv: torch.Tensor, nh: int, nkv: int, d: int, page_size: int, step,
-                      force: Optional[str], biased: bool = False, shaped: bool = False):
+                      force: Optional[str], biased: bool = False, shaped: bool = False,
+                      plain: bool = False):
     """(kind, matrix_decode): which attention kernel a batch takes.  A bias on the scores
     changes nothing here: every kernel takes one.  ``shaped`` (a scale per head, a cap on the
     scores): the matrix-core kernels take it when ``SHAPED_SCORES_MATRIX`` says so."""
     kind = force or FORCE_ATTENTION
-    matrix = not shaped or SHAPED_SCORES_MATRIX
+    matrix = (not shaped or SHAPED_SCORES_MATRIX) and not plain
     if kind is None:
         if step.all_decode and d % 8 == 0 and d <= 256 and (nh // nkv) * d <= 2048:
             kind = "decode"
@@ -894,9 +1034,11 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                    bias_slopes: Optional[torch.Tensor] = None,
                    counters: Optional[torch.Tensor] = None,
                    head_scales: Optional[torch.Tensor] = None,
-                   softcap: float = 0.0) -> torch.Tensor:
-    """``rope_kv_write`` followed by ``paged_attention`` (``head_scales`` and ``softcap`` as
-    there).  A decode batch that takes the
+                   softcap: float = 0.0, sinks: Optional[torch.Tensor] = None,
+                   keep_first: int = 0) -> torch.Tensor:
+    """``rope_kv_write`` followed by ``paged_attention`` (``head_scales``, ``softcap``, ``sinks``
+    and ``keep_first`` as there).  ``qkv`` may hold the queries alone (``(T, nh * d)``) when
+    nothing is written to the cache.  A decode batch that takes the
     matrix-core decode kernel does both in that kernel when the whole head is rotated
     (rotate-half) and is 64, 128 or 256 wide (or nothing is rotated); ``qkv`` is then left
     unrotated.  Under the same conditions a batch with portions of prompts leaves the queries
@@ -907,8 +1049,19 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     nh, nkv, d = num_heads, num_kv_heads, head_dim
     _rows_contig(qkv, "qkv")
     shaped = head_scales is not None or softcap > 0
+    more = dict(head_scales=head_scales, softcap=softcap, sinks=sinks, keep_first=keep_first)
     kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, None, bias_slopes is not None,
-                                   shaped)
+                                   shaped, PLAIN_EXTRAS and (sinks is not None
+                                                             or bool(keep_first and window)))
+    if qkv.shape[1] == nh * d and not write_kv:
+        # queries alone, keys and values are another layer's: rotate in place where there is a
+        # rotation (as a row of heads without keys and values), then attend
+        if cos is not None:
+            rope_kv_write(qkv, nh, 0, d, cos, sin, positions, None, None, None, page_size,
+                          write_kv=False, interleaved=interleaved)
+        return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
+                               scale, window, plan=plan, bias_slopes=bias_slopes,
+                               counters=counters, **more)
     fusable = cos is None or (2 * cos.shape[1] == d and d in (64, 128, 256) and not interleaved)
     whole_rows = qkv.shape[1] == (nh + 2 * nkv) * d
     if cos is not None and fusable and whole_rows and (mfma or kind == "prefill"):
@@ -921,8 +1074,7 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
             raise KernelError("rope_attention: a cache write needs slots")
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
-                               bias_slopes=bias_slopes, head_scales=head_scales,
-                               softcap=softcap,
+                               bias_slopes=bias_slopes, **more,
                                rope=(cos, sin, positions, slots if write_kv else None))
     if (kind == "prefill" and cos is not None and fusable and FUSE_ROPE_PREFILL and whole_rows
             and (_decode_mfma_ok(qkv, nh, nkv, d, page_size)
@@ -931,13 +1083,12 @@ def rope_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                       write_kv=write_kv, rotate_q=False)
         return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                                scale, window, plan=plan, counters=counters,
-                               bias_slopes=bias_slopes, head_scales=head_scales,
-                               softcap=softcap, rope=(cos, sin, positions, None))
+                               bias_slopes=bias_slopes, **more, rope=(cos, sin, positions, None))
     rope_kv_write(qkv, nh, nkv, d, cos, sin, positions, slots, k_pages, v_pages, page_size,
                   write_kv=write_kv, interleaved=interleaved)
     return paged_attention(qkv, nh, nkv, d, k_pages, v_pages, page_size, block_tables, step,
                            scale, window, plan=plan, bias_slopes=bias_slopes, counters=counters,
-                           head_scales=head_scales, softcap=softcap)
+                           **more)
 
 
 def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
@@ -948,7 +1099,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                     bias_slopes: Optional[torch.Tensor] = None,
                     counters: Optional[torch.Tensor] = None,
                     head_scales: Optional[torch.Tensor] = None,
-                    softcap: float = 0.0) -> torch.Tensor:
+                    softcap: float = 0.0, sinks: Optional[torch.Tensor] = None,
+                    keep_first: int = 0) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache -> ``(T, nh * d)``.
 
     ``qkv`` holds the rotated queries in its first ``nh * d`` columns; K and V of the new
@@ -965,6 +1117,10 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     ``head_scales`` (float32, one per query head): the head's scores are multiplied by its
     number on top of ``scale``; ``softcap`` c > 0: the scaled score becomes ``c * tanh(score /
     c)`` before bias and softmax.  Both are float32 arithmetic in every kernel.
+    ``sinks`` (float32, one per query head): the softmax's denominator also holds ``e^sink`` of
+    the head, once, unscaled, with no key and no value behind it.  ``keep_first`` n (with a
+    window): the first n keys of a sequence stay visible to every later query, at their own
+    positions, beside the window's keys.
     ``force`` names one of 'generic', 'decode', 'prefill' for tests.  ``rope`` (from
     ``rope_attention`` only): ``(cos, sin, positions, slots)`` for the matrix-core decode kernel
     to rotate and store the step's tokens itself; with portions of prompts in the batch
@@ -1013,8 +1169,17 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     if softcap < 0:
         raise KernelError("attention: the cap of the scores must be positive (0: none)")
     shaped = scales_ptr is not None or softcap > 0
+    sinks_ptr = None
+    if sinks is not None:
+        _check(sinks, "sinks", torch.float32, 1)
+        if sinks.numel() != nh or not sinks.is_contiguous():
+            raise KernelError(f"attention: {sinks.numel()} sinks for {nh} heads")
+        sinks_ptr = sinks.data_ptr()
+    kept = int(keep_first or 0) if win else 0
+    if kept < 0:
+        raise KernelError("attention: the count of kept first keys must not be negative")
     kind, mfma = _attention_kernel(qkv, nh, nkv, d, page_size, step, force, slopes_ptr is not None,
-                                   shaped)
+                                   shaped, PLAIN_EXTRAS and (sinks_ptr is not None or kept > 0))
     if rope is not None and not (mfma or (kind == "prefill" and rope[3] is None
                                           and rope[0] is not None)):
         raise KernelError("attention: only the matrix-core kernels rotate, and only the decode "
@@ -1024,7 +1189,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                  k_pages.data_ptr(), v_pages.data_ptr(), block_tables.data_ptr(), max_pages,
                  _i32(step.seq_of_token, "seq_of_token", T), _i32(step.positions, "positions", T),
                  T, nh, nkv, d, page_size, float(scale), win, slopes_ptr, scales_ptr, softcap,
-                 stream)
+                 sinks_ptr, kept, stream)
         return out
     if kind not in ("decode", "prefill"):
         raise KernelError(f"attention: unknown kernel '{kind}'")
@@ -1078,7 +1243,8 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
                      block_tables.data_ptr(), max_pages, _i32(step.ctx_lens, "ctx_lens", S), None,
                      S, nh, nkv, d, page_size, float(scale), win, depth, ap.DECODE_PART_KEYS,
-                     ap.DECODE_MAX_PARTS, slopes_ptr, scales_ptr, softcap, stream)
+                     ap.DECODE_MAX_PARTS, slopes_ptr, scales_ptr, softcap, sinks_ptr, kept,
+                     stream)
 
     if kind == "decode":
         if not step.all_decode:
@@ -1136,7 +1302,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         lib.call("rlis_attn_reduce_rows", out.data_ptr(), nh * d, ml_ptr, acc_ptr,
                  _i32(step.seq_of_token, "seq_of_token", T),
                  _i32(plan["seq_runs"], "seq_runs", step.num_seqs), row0, T - row0, nh, d,
-                 max_runs, stream)
+                 max_runs, sinks_ptr, stream)
     return out
 
 

@@ -19,6 +19,10 @@ P, I, L, F = c_void_p, c_int, c_longlong, c_float
 _SIGNATURES = {
     "rlis_embed": [P, P, I, P, I, I, F, P, P, P],
     "rlis_gelu_tanh": [P, P, I, L, P],
+    "rlis_gelu_erf": [P, P, I, L, P],
+    "rlis_lanes_step": [P, L, P, L, P, I, I, L, I, P, P, P, P, I, F, P, I, P, I, I, I, I, P],
+    "rlis_head_prepare": [P, I, L, I, I, I, I, I, P, P, P, F, P, F, I, P],
+    "rlis_head_gate": [P, I, L, P, L, I, I, I, P],
     "rlis_depth_mix": [P, P, P, L, I, P, I, I, P],
     "rlis_decay_attention_scan": [P, P, L, P, L, P, L, I, P, P, L, P, P, I, I, I, I, I, I, P],
     "rlis_decay_attention_chunks": [P, P, L, P, L, P, L, P, P, L, P, P, I, I, I, I, I, I, P, I, P],
@@ -41,7 +45,7 @@ _SIGNATURES = {
     "rlis_latent_attention": [P, I, L, P, L, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_sigmoid_gate": [P, L, P, L, I, I, I, P],
     "rlis_moe_router_logits": [P, P, P, F, P, I, P, I, I, I, P],
-    "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, I, I, I, P],
+    "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, I, I, I, P, P],
     "rlis_moe_sort": [P, I, I, I, I, P, P, P],
     "rlis_moe_experts": [P, I, L, P, P, P, P, P, I, I, I, I, I, P, P, F, F, P],
     "rlis_moe_combine": [P, P, P, I, I, I, I, P],
@@ -59,13 +63,14 @@ _SIGNATURES = {
     "rlis_gemm_bf16_stream_join": [P, P, I, I, I, L, L, P, P, P, I, I, P, P, I, P],
     "rlis_gemm_bf16_stream_scaled": [P, P, P, I, I, I, I, L, L, L, I, P, I, I, F, P],
     "rlis_norm_linear_bf16": [P, P, I, I, L, I, P, I, F, P, P, P, P, I, I, I, I, L, L, I, P],
-    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P, F, P],
-    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P, F, P],
+    "rlis_attn_generic": [P, I, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, P, P, F, P, I, P],
+    "rlis_attn_decode": [P, I, L, P, L, P, P, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, I, P, P, F,
+                         P, I, P],
     "rlis_attn_decode_mfma": [P, L, P, L, P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, I, I, P, I, I, I,
                               P, P, I, P, P, L, L, P, P, F, P],
     "rlis_attn_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, I, P, P,
                                P, P, I, P, P, F, P],
-    "rlis_attn_reduce_rows": [P, L, P, P, P, P, I, I, I, I, I, P],
+    "rlis_attn_reduce_rows": [P, L, P, P, P, P, I, I, I, I, I, P, P],
     "rlis_sample_rows": [P, L, I, I, P, P, P, I, P, P, P],
     "rlis_fill_normal_device": [P, I, L, ctypes.c_ulonglong, ctypes.c_ulonglong, ctypes.c_double,
                                 ctypes.c_double, P],

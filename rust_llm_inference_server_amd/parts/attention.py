@@ -40,6 +40,24 @@ class PagedAttention(Mixer):
       The source layer hands its values (behind the convolution) on to the later layers of the
       step under ``key``; every other layer with that key replaces its values by
       ``(1 - w) v + w v_source`` (``w`` the tensor's one number) before they are cached.
+    * ``bias``: a suffix; the q, k and v projections add the tensors ``<q|k|v name><suffix>``
+      (one number per output column, float32 arithmetic on the stored product).
+    * ``qk_norm``: ``{"q": name, "k": name, "eps": e}``.  Every query head and every key head is
+      divided by the root mean square of its own numbers (eps inside the root) and multiplied by
+      the named weight of ``head_dim`` numbers, which all heads share, behind the bias and in
+      front of the rotation; the cache holds the normalised keys.
+    * ``query_temperature``: ``{"coef": c, "every": n}``.  The queries of a token at position p
+      are multiplied by ``1 + c ln(floor((p + 1) / n) + 1)`` (behind the norm).
+    * ``sinks``: the name of a tensor with one number per query head: the softmax's denominator
+      also holds ``e^sink``, once, unscaled, with no key and no value behind it.
+    * ``keep_first`` n (with a ``window``): the first n keys of a sequence stay visible to every
+      later query beside the window's keys, at their own positions.  The cache then keeps every
+      position of such a layer.
+    * ``gate``: the name of a projection ``(num_heads, hidden_size)`` of the mixer's input: head
+      h of the result is multiplied by the sigmoid of output h, in front of the output
+      projection.
+    * ``shared_kv``: the layer has no key and value projections (nor what belongs to them:
+      biases, the keys' norm); its run reads the cache that another run wrote.
 
     With ``value_dim != head_dim`` (or an odd head size) the kernels run at one head size ``D``,
     the larger of the two rounded up to a multiple of 16: the rows of the narrower projection's weight are padded
@@ -68,8 +86,22 @@ class PagedAttention(Mixer):
                                              "head_dim"))
         dv = params.get("value_dim") or d
         n = cls._names(params, prefix)
-        out = [TensorSpec(n["q"], (nh * d, H)), TensorSpec(n["k"], (nkv * d, H)),
-               TensorSpec(n["v"], (nkv * dv, H)), TensorSpec(n["o"], (H, nh * dv))]
+        own_kv = not params.get("shared_kv")
+        out = [TensorSpec(n["q"], (nh * d, H))]
+        if own_kv:
+            out += [TensorSpec(n["k"], (nkv * d, H)), TensorSpec(n["v"], (nkv * dv, H))]
+        out.append(TensorSpec(n["o"], (H, nh * dv)))
+        if params.get("bias"):
+            out += [TensorSpec(n[c] + params["bias"], (rows,), std=0.1) for c, rows in
+                    (("q", nh * d), ("k", nkv * d), ("v", nkv * dv)) if c == "q" or own_kv]
+        norm = params.get("qk_norm")
+        if norm:
+            out += [TensorSpec(join(prefix, norm[c]), (d,), init="ones_normal", std=0.1)
+                    for c in "qk" if c == "q" or own_kv]
+        if params.get("sinks"):
+            out.append(TensorSpec(join(prefix, params["sinks"]), (nh,), std=1.0))
+        if params.get("gate"):
+            out.append(TensorSpec(join(prefix, params["gate"]), (nh, H), std=0.1))
         taps = params.get("conv")
         if taps:
             out += [TensorSpec(n[c] + ".conv", (rows, int(taps)), std=0.3)
@@ -112,15 +144,49 @@ class PagedAttention(Mixer):
             raise ValueError(f"attention: {self.num_heads} heads are not a multiple of "
                              f"{self.num_kv_heads} KV heads")
         names = self._names(params, prefix)
-        q, k, v = (ctx.weights.pop(names[n]) for n in "qkv")
-        if not (q.dtype == k.dtype == v.dtype):
-            q, k, v = (t.to(torch.float32) for t in (q, k, v))
-        q = self._pad_heads(q, self.num_heads, qk_dim, self.head_dim, rows=True)
-        k = self._pad_heads(k, self.num_kv_heads, qk_dim, self.head_dim, rows=True)
-        v = self._pad_heads(v, self.num_kv_heads, v_dim, self.head_dim, rows=True)
-        # One product for q, k and v: the rows of the three weights, concatenated.
-        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
-        del q, k, v
+        self.shared_kv = bool(params.get("shared_kv"))
+        self.qk_dim = qk_dim
+        # (heads, real size) of the projections this layer has, in the order of the row
+        kinds = [("q", self.num_heads, qk_dim)]
+        if not self.shared_kv:
+            kinds += [("k", self.num_kv_heads, qk_dim), ("v", self.num_kv_heads, v_dim)]
+        mats = [ctx.weights.pop(names[c]) for c, _, _ in kinds]
+        gate = ctx.weights.pop(join(prefix, params["gate"])) if params.get("gate") else None
+        if len({t.dtype for t in mats + ([gate] if gate is not None else [])}) > 1:
+            mats = [t.to(torch.float32) for t in mats]
+            gate = None if gate is None else gate.to(torch.float32)
+        mats = [self._pad_heads(t, heads, size, self.head_dim, rows=True)
+                for t, (_, heads, size) in zip(mats, kinds)]
+        # the columns of q, k and v in the product's rows
+        self.qkv_cols = sum(t.shape[0] for t in mats)
+        self.gated = gate is not None
+        if gate is not None:
+            # the gates' rows ride behind v, padded so that rows stay 16-byte aligned
+            pad = -gate.shape[0] % 8
+            mats.append(torch.cat([gate, gate.new_zeros((pad, gate.shape[1]))], dim=0))
+        # One product for q, k and v (and the gates): the rows of the weights, concatenated.
+        self.w_qkv = torch.cat(mats, dim=0).contiguous()
+        del mats, gate
+        self.bias = None
+        if params.get("bias"):
+            self.bias = torch.cat([
+                self._pad_heads(ctx.take(names[c] + params["bias"]).to(torch.float32).reshape(-1, 1),
+                                heads, size, self.head_dim, rows=True).reshape(-1)
+                for c, heads, size in kinds]).contiguous()
+        self.q_norm = self.k_norm = None
+        self.norm_eps = 0.0
+        norm = params.get("qk_norm")
+        if norm:
+            self.norm_eps = float(norm["eps"])
+            self.q_norm = ctx.take(join(prefix, norm["q"])).to(torch.float32).contiguous()
+            if not self.shared_kv:
+                self.k_norm = ctx.take(join(prefix, norm["k"])).to(torch.float32).contiguous()
+        temp = params.get("query_temperature") or {}
+        self.temp_coef, self.temp_every = float(temp.get("coef", 0.0)), int(temp.get("every", 0))
+        self.sinks = None
+        if params.get("sinks"):
+            self.sinks = ctx.take(join(prefix, params["sinks"])).to(torch.float32).contiguous()
+        self.keep_first = int(params.get("keep_first") or 0)
         self.w_o = self._pad_heads(ctx.take(names["o"]), self.num_heads, v_dim, self.head_dim,
                                    rows=False).contiguous()
         self.act_dtype = ctx.act_dtype
@@ -135,6 +201,9 @@ class PagedAttention(Mixer):
             if not 1 <= self.taps <= 16:
                 raise ValueError(f"attention: {self.taps} taps (1 to 16)")
             # the taps of every channel of the one product, padded channels with zero taps
+            if self.shared_kv or self.gated:
+                raise ValueError("attention: the convolutions are built for layers with q, k and "
+                                 "v projections of their own and no gate")
             pads = ((names["q"], nh, qk_dim), (names["k"], nkv, qk_dim), (names["v"], nkv, v_dim))
             self.conv_w = torch.cat([
                 self._pad_heads(ctx.take(n + ".conv").to(torch.float32), heads, size, D, rows=True)
@@ -157,10 +226,13 @@ class PagedAttention(Mixer):
         self.planner = ops.attention_planner(
             self.num_heads, self.num_kv_heads, self.head_dim, self.act_dtype,
             biased=getattr(self.position, "bias_slopes", None) is not None,
-            shaped=self.head_scales is not None or self.softcap > 0)
+            shaped=self.head_scales is not None or self.softcap > 0,
+            plain=self.sinks is not None or bool(self.keep_first and self.window))
 
     def cache_request(self) -> CacheRequest:
-        return CacheRequest.kv(self.num_kv_heads, self.head_dim, self.window)
+        # (first keys that stay visible: the pages behind the window are not given back)
+        window = None if self.keep_first else self.window
+        return CacheRequest.kv(self.num_kv_heads, self.head_dim, window)
 
     def step_planner(self):
         return self.planner
@@ -177,6 +249,10 @@ class PagedAttention(Mixer):
         has them."""
         if not self.taps:
             qkv = project(x, self.w_qkv, self.act_dtype)
+            if self.bias is not None or self.q_norm is not None or self.temp_every:
+                ops.head_prepare_(qkv, self.num_heads, 0 if self.shared_kv else self.num_kv_heads,
+                                  self.head_dim, self.qk_dim, self.bias, self.q_norm, self.k_norm,
+                                  self.norm_eps, step.positions, self.temp_coef, self.temp_every)
         else:
             C = self.w_qkv.shape[0]
             if isinstance(x, NormedInput) and not ops.can_fuse_norm_linear(
@@ -220,7 +296,11 @@ class PagedAttention(Mixer):
 
     def forward(self, x: Any, step: Any, binding: CacheBinding) -> torch.Tensor:
         group = step.groups[binding.group]
-        qkv = self._project(x, step, binding)
+        if self.shared_kv and binding.writes:
+            raise ValueError("attention: a layer without keys and values of its own must read "
+                             "another run's cache")
+        rows = self._project(x, step, binding)
+        qkv = rows[:, :self.qkv_cols] if self.gated else rows
         if step.max_context > self.position.max_positions:
             raise ValueError(f"sequence of {step.max_context} positions exceeds max_seq_len "
                              f"{self.position.max_positions}")
@@ -228,9 +308,13 @@ class PagedAttention(Mixer):
                                  self.position.cos, self.position.sin, step.positions,
                                  group.slots, binding.k_pages, binding.v_pages, group.page_size,
                                  group.block_tables, step, self.scale, self.window,
-                                 write_kv=binding.writes, plan=step.plans.get(self.planner.key()),
+                                 write_kv=binding.writes and not self.shared_kv,
+                                 plan=step.plans.get(self.planner.key()),
                                  interleaved=bool(getattr(self.position, "interleaved", False)),
                                  bias_slopes=getattr(self.position, "bias_slopes", None),
                                  counters=binding.counters, head_scales=self.head_scales,
-                                 softcap=self.softcap)
+                                 softcap=self.softcap, sinks=self.sinks,
+                                 keep_first=self.keep_first)
+        if self.gated:
+            ops.head_gate_(out, rows[:, self.qkv_cols:], self.num_heads, self.head_dim)
         return ops.pending_linear(out, self.w_o, self.act_dtype)

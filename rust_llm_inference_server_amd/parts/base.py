@@ -369,6 +369,60 @@ def as_tensor(delta: Any) -> torch.Tensor:
     return delta.sum(0) if delta.dim() == 3 else delta
 
 
+class LaneSet:
+    """Several residual streams side by side (hyper-connections): ``count`` float32 tensors
+    ``(T, H)`` that start out equal to the stream they were made from.  A sublayer reads a
+    weighted sum of them through its norm (``reading`` names the weights of the next read),
+    and its result comes back into all of them at once: ``update(y, mix, back)`` leaves
+    ``lanes'[t] = sum_s mix[s, t] lanes[s] + back[t] y`` *pending*, so that the next read does
+    the update and the read in one pass (``ops.lanes_step``).  ``total()`` is the plain sum of
+    the streams."""
+
+    __slots__ = ("count", "lanes", "pending", "read", "round_parts")
+
+    def __init__(self, x: torch.Tensor, count: int, round_parts: bool):
+        self.count = int(count)
+        self.lanes = x                 # (T, H) while all streams are equal, then (count, T, H)
+        self.pending: Any = None       # (y, mix, back)
+        self.read: Optional[torch.Tensor] = None
+        self.round_parts = round_parts
+
+    def reading(self, weights: Optional[torch.Tensor]) -> None:
+        self.read = weights
+
+    def update(self, y: Any, mix: torch.Tensor, back: torch.Tensor) -> None:
+        if self.pending is not None:
+            self.settle()
+        if not isinstance(y, torch.Tensor):
+            y = y.run()
+        self.pending = (y, mix, back)
+
+    def settle(self) -> None:
+        from .. import ops
+        if self.pending is not None:
+            self.lanes, _ = ops.lanes_step(self.lanes, self.count, update=self.pending,
+                                           round_parts=self.round_parts, want=False)
+            self.pending = None
+
+    def normed(self, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+               rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The pending update, then the read-out through the norm (``weight`` None: as it is,
+        float32).  With ``rows`` only those tokens, and the streams stay as they are."""
+        from .. import ops
+        lanes, out = ops.lanes_step(self.lanes, self.count, update=self.pending, read=self.read,
+                                    norm_weight=weight, eps=eps, out_dtype=out_dtype, rows=rows,
+                                    round_parts=self.round_parts)
+        if rows is None:
+            self.lanes, self.pending = lanes, None
+        return out
+
+    def total(self) -> torch.Tensor:
+        self.reading(None)
+        if self.lanes.dim() == 2 and self.pending is None:
+            return self.lanes * float(self.count) if self.count != 1 else self.lanes
+        return self.normed(None, 0.0, torch.float32)
+
+
 class ResidualStream:
     """The residual sum, kept in 32-bit, plus a delta that has not been added yet.
 
@@ -379,7 +433,7 @@ class ResidualStream:
     (``round_parts``), as a delta that arrives whole in bfloat16 was by its kernel, so that the
     rounding does not depend on which kernel a batch's size chose."""
 
-    __slots__ = ("x", "pending", "pending_scale", "round_parts", "history")
+    __slots__ = ("x", "pending", "pending_scale", "round_parts", "history", "lanes")
 
     def __init__(self, x: torch.Tensor, act_dtype: torch.dtype = torch.float32):
         assert x.dtype == torch.float32
@@ -394,6 +448,23 @@ class ResidualStream:
         # (slots, T, H) float32: the embedding output and the layers' results so far, for
         # blocks that feed the next layer a mix of them (made by the first such block)
         self.history: Optional[torch.Tensor] = None
+        # several streams in place of ``x`` (made by the first block that keeps them); norms
+        # read them through ``LaneSet.normed``, ``merge_lanes`` makes ``x`` their sum again
+        self.lanes: Optional[LaneSet] = None
+
+    def split_lanes(self, count: int) -> LaneSet:
+        """``count`` streams that all start as the residual sum; ``x`` is theirs from now on."""
+        if self.lanes is None:
+            self.lanes = LaneSet(self.flush(), count, self.round_parts)
+        elif self.lanes.count != count:
+            raise ValueError(f"the step keeps {self.lanes.count} residual streams, a block "
+                             f"asks for {count}")
+        return self.lanes
+
+    def merge_lanes(self) -> None:
+        """One stream again: the sum of the streams."""
+        if self.lanes is not None:
+            self.x, self.lanes = self.lanes.total(), None
 
     def add(self, delta: Any, scale: float = 1.0) -> None:
         if self.pending is not None:

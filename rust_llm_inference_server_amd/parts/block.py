@@ -62,6 +62,64 @@ class PreNormBlock(Block):
                 normed(self.ffn_norm, stream, self.feed_forward), step), m)
 
 
+@register("block", "hyper")
+class HyperBlock(PreNormBlock):
+    """The pre-norm block over several residual streams (hyper-connections).  In place of one
+    x there are ``streams`` copies x_1 .. x_S, all equal to the block's input stream when the
+    first such block meets it.  Sublayer q (1: the mixer, 2: the feed-forward) reads
+    ``u = sum_s in_q[s] x_s`` through its norm, and its result y comes back into all streams at
+    once, from the old ones: ``x_t <- sum_s mix_q[s, t] x_s + out_q[t] y``.
+
+    Parameters: those of ``prenorm`` (without ``residual_scale``), ``streams`` and ``connections``:
+    the tensors' prefixes under the block's prefix, one per sublayer (``("hc1", "hc2")``), each
+    with ``.in`` (S), ``.out`` (S) and ``.mix`` (S, S, indexed [from, to]).  ``last``: the block
+    leaves one stream behind, the sum of the S, for blocks of another kind behind it (a norm
+    behind the last block reads that sum from the streams by itself).  The streams,
+    the coefficients and every sum are float32; update and next read run as one kernel."""
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        out = super().tensor_specs(params, prefix)
+        S = int(params["streams"])
+        subs = 1 if params.get("feed_forward") is None else 2
+        for name in tuple(params["connections"])[:subs]:
+            base = join(prefix, name)
+            out += [TensorSpec(base + ".in", (S,), init="ones_normal", std=0.2),
+                    TensorSpec(base + ".out", (S,), init="ones_normal", std=0.2),
+                    TensorSpec(base + ".mix", (S, S), std=0.4)]
+        return out
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        if self.residual_scale != 1.0:
+            raise ValueError("block 'hyper': the streams' own coefficients scale the results")
+        self.streams = int(params["streams"])
+        self.last = bool(params.get("last"))
+        subs = 1 if self.feed_forward is None else 2
+        take = lambda n: ctx.take(n).to(torch.float32).contiguous()
+        self.connections = [tuple(take(join(prefix, name) + part) for part in (".in", ".mix", ".out"))
+                            for name in tuple(params["connections"])[:subs]]
+        for read, mix, back in self.connections:
+            if read.numel() != self.streams or back.numel() != self.streams \
+                    or tuple(mix.shape) != (self.streams, self.streams):
+                raise ValueError(f"block 'hyper': coefficients do not fit {self.streams} streams")
+
+    def forward(self, stream: ResidualStream, step: Any, binding: CacheBinding) -> None:
+        lanes = stream.split_lanes(self.streams)
+        read, mix, back = self.connections[0]
+        lanes.reading(read)
+        lanes.update(self.mixer.forward(normed(self.mixer_norm, stream, self.mixer), step, binding),
+                     mix, back)
+        if self.feed_forward is not None:
+            read, mix, back = self.connections[1]
+            lanes.reading(read)
+            lanes.update(self.feed_forward.forward(
+                normed(self.ffn_norm, stream, self.feed_forward), step), mix, back)
+        lanes.reading(None)          # whoever reads next without weights reads the plain sum
+        if self.last:
+            stream.merge_lanes()
+
+
 @register("block", "parallel")
 class ParallelBlock(Block):
     """Parameters: ``mixer``, ``feed_forward`` (None: the mixer alone), ``norm`` (PartSpecs) and

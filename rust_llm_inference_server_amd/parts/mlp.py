@@ -54,7 +54,8 @@ class DenseMLP(FeedForward):
     graph_safe = True
     takes_normed_input = True        # the norm in front goes into the up product where it can
 
-    ACTIVATIONS = {"gelu_tanh": "gelu_tanh"}       # activation -> the kernel's name in ops
+    # activation -> the kernel's name in ops ("gelu_erf": 0.5 z (1 + erf(z / sqrt 2)))
+    ACTIVATIONS = {"gelu_tanh": "gelu_tanh", "gelu_erf": "gelu_erf"}
 
     @classmethod
     def _names(cls, params: Dict[str, Any], prefix: str) -> Dict[str, str]:
@@ -233,3 +234,62 @@ class RoutedSwiGLU(FeedForward):
                                 self.act_dtype)
         return ops.routed_units(x, self.w_gate_up, self.w_down, chosen, weights, shared,
                                 limit=self.limit, alpha=self.alpha)
+
+
+@register("feed_forward", "routed_mlp")
+class RoutedMLP(FeedForward):
+    """A mixture of small two-projection units ``down(act(up(x)))`` without gates, of which
+    every token takes the ``top`` with the largest router logits; their weights are the softmax
+    over the chosen logits alone.
+
+    Parameters: ``hidden_size``, ``expert_size`` (an expert's inner width), ``experts``, ``top``,
+    ``activation`` ("relu2": the square of ReLU), ``router_bias`` (the suffix of the bias tensor
+    behind the router's name, None: no bias).  Tensors under the prefix: ``router`` (experts, W),
+    ``router<suffix>`` (experts), ``e<i>.up`` (F, W), ``e<i>.down`` (W, F).  Router logits, the
+    choice and the weights are float32; the logits are the product of the activations as the
+    experts read them."""
+
+    graph_safe = True
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        W, F, E = params["hidden_size"], params["expert_size"], params["experts"]
+        out: List[TensorSpec] = []
+        for e in range(E):
+            out += [TensorSpec(join(prefix, f"e{e}.up"), (F, W)),
+                    TensorSpec(join(prefix, f"e{e}.down"), (W, F))]
+        out += [TensorSpec(join(prefix, "router"), (E, W), std=0.5)]
+        if params.get("router_bias"):
+            out += [TensorSpec(join(prefix, "router") + params["router_bias"], (E,), std=0.1)]
+        return out
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        E = self.experts = int(params["experts"])
+        self.top = int(params["top"])
+        if params.get("activation", "relu2") != "relu2":
+            raise ValueError(f"routed_mlp: activation '{params['activation']}' is not known "
+                             "(known: 'relu2')")
+        if not 1 <= self.top <= E:
+            raise ValueError(f"routed_mlp: {self.top} chosen of {E} experts")
+        self.act_dtype = ctx.act_dtype
+        pop = lambda n: ctx.weights.pop(join(prefix, n)).to(ctx.act_dtype)
+        up = torch.stack([pop(f"e{e}.up") for e in range(E)])
+        down = torch.stack([pop(f"e{e}.down") for e in range(E)])
+        if up.shape[1] % 2:
+            # the kernels take the inner width in two halves: one more unit that is always zero
+            up = torch.cat([up, up.new_zeros((E, 1, up.shape[2]))], dim=1)
+            down = torch.cat([down, down.new_zeros((E, down.shape[1], 1))], dim=2)
+        self.w_up, self.w_down = up.contiguous(), down.contiguous()
+        self.w_router = ctx.take(join(prefix, "router"))
+        self.router_bias = None
+        if params.get("router_bias"):
+            self.router_bias = ctx.take(join(prefix, "router") + params["router_bias"]).to(
+                torch.float32).contiguous()
+
+    def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
+        logits = ops.linear(x, self.w_router, torch.float32)
+        # softmax over all experts, renormalised over the chosen: the softmax over the chosen
+        chosen, weights = ops.route(logits, None, 1, 1, self.top, 1.0, scores="softmax",
+                                    group_score="max", renormalise=True, bias=self.router_bias)
+        return ops.routed_units(x, self.w_up, self.w_down, chosen, weights, plain=True)

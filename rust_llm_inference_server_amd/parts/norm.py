@@ -51,18 +51,22 @@ class RMSNorm(Norm):
         self.out_dtype = ctx.act_dtype
 
     def forward(self, stream: ResidualStream) -> torch.Tensor:
+        if stream.lanes is not None:
+            return stream.lanes.normed(self.weight, self.eps, self.out_dtype)
         delta, scale = stream.take_delta()
         return ops.add_rmsnorm(stream.x, delta, self.weight, self.eps, self.out_dtype,
                                round_parts=stream.round_parts, delta_scale=scale)
 
     def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
+        if stream.lanes is not None:
+            return stream.lanes.normed(self.weight, self.eps, self.out_dtype, rows)
         return ops.add_rmsnorm(stream.x, stream.delta(), self.weight, self.eps, self.out_dtype,
                                rows=rows, round_parts=stream.round_parts,
                                delta_scale=stream.pending_scale)
 
     def fused_linear(self, stream: ResidualStream, w: torch.Tensor, out_dtype: torch.dtype,
                      gated: bool, rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
-        if self.out_dtype != torch.bfloat16:
+        if self.out_dtype != torch.bfloat16 or stream.lanes is not None:
             return None
         if stream.pending is not None and stream.pending_scale != 1.0:
             if rows is not None:

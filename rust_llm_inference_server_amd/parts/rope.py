@@ -67,8 +67,9 @@ def inverse_frequencies(rot_dim: int, theta: float, scaling: Optional[Dict[str, 
 @register("position", "rope")
 class RotaryEmbedding(PositionEncoding):
     """Parameters: ``rot_dim`` (rotated width, at most the head size), ``theta``, ``scaling``
-    (None, the llama3 fields, or ``{"rope_type": "yarn", "factor", "original", "fast",
-    "slow"}``).  Holds ``cos``/``sin`` float32 ``(max_positions, rot/2)``.
+    (None, the llama3 fields, ``{"rope_type": "yarn", "factor", "original", "fast",
+    "slow"}``, or with ``precise`` ``{"rope_type": "linear", "factor"}``: every frequency divided
+    by the factor).  Holds ``cos``/``sin`` float32 ``(max_positions, rot/2)``.
     Optional ``precise``: frequencies, angles, cosines and sines are made in double precision
     and rounded once to float32 (without it they are float32 from the start, as the reference
     makes them); yarn scaling is always made that way."""
@@ -85,10 +86,17 @@ class RotaryEmbedding(PositionEncoding):
             magnitude = 0.1 * math.log(float(scaling["factor"])) + 1.0
             pos = torch.arange(ctx.max_positions, dtype=torch.float64).reshape(-1, 1)
         elif params.get("precise"):
-            if scaling:
+            if scaling and scaling.get("rope_type") != "linear":
                 raise ValueError("position encoding 'rope': 'precise' has no llama3 scaling")
             f64 = torch.float64
             inv = float(params["theta"]) ** (-torch.arange(0, rot, 2, dtype=f64) / rot)
+            if scaling:
+                # positions stretched evenly: every frequency divided by the factor
+                factor = float(scaling.get("factor") or 0.0)
+                if not factor > 0:
+                    raise ValueError("position encoding 'rope': linear scaling needs a positive "
+                                     "'factor'")
+                inv = inv / factor
             pos = torch.arange(ctx.max_positions, dtype=f64).reshape(-1, 1)
         else:
             inv = inverse_frequencies(rot, params["theta"], params.get("scaling"))

@@ -22,6 +22,58 @@ def gelu_tanh(x):
     return (0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))).to(x.dtype)
 
 
+def gelu_erf(x):
+    z = x.float()
+    return (0.5 * z * (1.0 + torch.erf(z * 0.7071067811865476))).to(x.dtype)
+
+
+def lanes_step(lanes, count, update=None, read=None, norm_weight=None, eps=0.0, out_dtype=None,
+               rows=None, round_parts=False, want=True):
+    S = count
+    cur = lanes.unsqueeze(0).expand(S, *lanes.shape) if lanes.dim() == 2 else lanes
+    if update is not None:
+        y, mix, back = update
+        y = (y.sum(0) if y.dim() == 3 else y).float()
+        cur = torch.stack([sum(mix[s, t] * cur[s] for s in range(S)) + back[t] * y
+                           for t in range(S)])
+    out = None
+    if want:
+        pick = cur if rows is None else cur[:, rows.long()]
+        u = sum((1.0 if read is None else read[s]) * pick[s] for s in range(S))
+        if norm_weight is not None:
+            u = u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        out = u.to(out_dtype or torch.float32)
+    keep = update is not None and rows is None
+    return (cur.contiguous() if keep else lanes), out
+
+
+def head_prepare_(qkv, num_heads, num_kv_heads, head_dim, real_dim, bias=None, q_weight=None,
+                  k_weight=None, eps=0.0, positions=None, temp_coef=0.0, temp_every=0):
+    T, nh, nkv, D = qkv.shape[0], num_heads, num_kv_heads, head_dim
+    cols = (nh + 2 * nkv) * D
+    x = qkv[:, :cols].float()
+    if bias is not None:
+        x = x + bias
+    x = x.reshape(T, nh + 2 * nkv, D).clone()
+    for lo, hi, w in ((0, nh, q_weight), (nh, nh + nkv, k_weight)):
+        if w is not None and hi > lo:
+            part = x[:, lo:hi, :real_dim]
+            x[:, lo:hi, :real_dim] = part / torch.sqrt((part * part).mean(-1, keepdim=True) + eps) * w
+            x[:, lo:hi, real_dim:] = 0.0
+    if temp_every > 0:
+        steps = torch.div(positions.long() + 1, temp_every, rounding_mode="floor").float()
+        x[:, :nh] = x[:, :nh] * (1.0 + temp_coef * torch.log(steps + 1.0)).reshape(T, 1, 1)
+    qkv[:, :cols] = x.reshape(T, cols).to(qkv.dtype)
+    return qkv
+
+
+def head_gate_(x, gate, num_heads, head_dim):
+    T = x.shape[0]
+    g = torch.sigmoid(gate[:, :num_heads].float()).reshape(T, num_heads, 1)
+    x.copy_((x.float().reshape(T, num_heads, head_dim) * g).reshape(T, -1).to(x.dtype))
+    return x
+
+
 def depth_mix_(x, delta, history, count, weights, save_input=False):
     if save_input:
         history[0] = x
@@ -253,8 +305,10 @@ def router_logits(resid, norm_weight, norm_bias, eps, w_router):
 
 
 def route(logits, correction, groups, keep, top, scale, scores="sigmoid", group_score="top2",
-          renormalise=False):
+          renormalise=False, bias=None):
     T, E = logits.shape
+    if bias is not None:
+        logits = logits + bias
     s = torch.sigmoid(logits) if scores == "sigmoid" else torch.softmax(logits, dim=-1)
     choice = (s if correction is None else s + correction).reshape(T, groups, E // groups)
     score = choice.topk(1 if group_score == "max" else min(2, E // groups), dim=-1).values.sum(-1)
@@ -268,14 +322,17 @@ def route(logits, correction, groups, keep, top, scale, scores="sigmoid", group_
     return chosen.to(torch.int32), weights
 
 
-def routed_units(x, w_gate_up, w_down, chosen, weights, addend=None, limit=0.0, alpha=1.0):
+def routed_units(x, w_gate_up, w_down, chosen, weights, addend=None, limit=0.0, alpha=1.0,
+                 plain=False):
     T, W = x.shape
     F = w_gate_up.shape[1] // 2
     out = torch.zeros(T, W)
     for t in range(T):
         for e, wt in zip(chosen[t].tolist(), weights[t].tolist()):
             gu = w_gate_up[e].float() @ x[t].float()
-            if limit > 0:
+            if plain:
+                hidden = (gu.clamp(min=0.0) ** 2).to(x.dtype).float()
+            elif limit > 0:
                 g, u = gu[:F].clamp(max=limit), gu[F:].clamp(-limit, limit)
                 hidden = (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(x.dtype).float()
             else:
@@ -355,7 +412,7 @@ def rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, s
     x = qkv.float()
     q = x[:, :nh * d].reshape(T, nh, d).clone()
     k = x[:, nh * d:(nh + nkv) * d].reshape(T, nkv, d).clone()
-    v = x[:, (nh + nkv) * d:].reshape(T, nkv, d)
+    v = x[:, (nh + nkv) * d:(nh + 2 * nkv) * d].reshape(T, nkv, d)
     if cos is not None:
         half = cos.shape[1]
         c = cos[positions.long()].unsqueeze(1)
@@ -377,14 +434,16 @@ def copy_pages(pages, src, dst):
         pages[:, d] = pages[:, s]
 
 
-def attention_planner(num_heads, num_kv_heads, head_dim, dtype, biased=False, shaped=False):
+def attention_planner(num_heads, num_kv_heads, head_dim, dtype, biased=False, shaped=False,
+                      plain=False):
     from rust_llm_inference_server_amd.ops.attention_plan import AttentionPlanner
     return AttentionPlanner(num_heads, num_kv_heads, head_dim, matrix=dtype == torch.bfloat16)
 
 
 def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
                     block_tables, step, scale, window=None, force=None, plan=None,
-                    bias_slopes=None, counters=None, head_scales=None, softcap=0.0):
+                    bias_slopes=None, counters=None, head_scales=None, softcap=0.0, sinks=None,
+                    keep_first=0):
     assert bias_slopes is None, "the test double adds no bias"
     T = qkv.shape[0]
     nh, nkv, d = num_heads, num_kv_heads, head_dim
@@ -396,7 +455,7 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
     for t in range(T):
         table = block_tables[seq_of[t]].tolist()
         lo = max(0, pos[t] - window + 1) if window else 0
-        keys = list(range(lo, pos[t] + 1))
+        keys = list(range(0, min(keep_first, lo) if window else 0)) + list(range(lo, pos[t] + 1))
         k = torch.stack([k_pages[table[p // page_size], :, p % page_size, :] for p in keys]).float()
         v = torch.stack([v_pages[table[p // page_size], :, :, p % page_size] for p in keys]).float()
         for h in range(nh):
@@ -405,7 +464,10 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
                 s = s * head_scales[h]
             if softcap:
                 s = softcap * torch.tanh(s / softcap)
-            p = torch.softmax(s, dim=0)
+            if sinks is not None:
+                p = torch.softmax(torch.cat([s, sinks[h].reshape(1).float()]), dim=0)[:-1]
+            else:
+                p = torch.softmax(s, dim=0)
             out[t, h * d:(h + 1) * d] = p @ v[:, h // g, :]
     return out.to(qkv.dtype)
 
@@ -413,12 +475,13 @@ def paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, pa
 def rope_attention(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
                    v_pages, page_size, block_tables, step, scale, window=None, write_kv=True,
                    plan=None, interleaved=False, bias_slopes=None, counters=None,
-                   head_scales=None, softcap=0.0):
-    rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, cos, sin, positions, slots, k_pages,
-                  v_pages, page_size, write_kv=write_kv)
+                   head_scales=None, softcap=0.0, sinks=None, keep_first=0):
+    own = 0 if qkv.shape[1] == num_heads * head_dim else num_kv_heads     # queries alone?
+    rope_kv_write(qkv, num_heads, own, head_dim, cos, sin, positions, slots, k_pages,
+                  v_pages, page_size, write_kv=write_kv and own > 0)
     return paged_attention(qkv, num_heads, num_kv_heads, head_dim, k_pages, v_pages, page_size,
                            block_tables, step, scale, window, head_scales=head_scales,
-                           softcap=softcap)
+                           softcap=softcap, sinks=sinks, keep_first=keep_first)
 
 
 def _lowbias32(x):
@@ -460,6 +523,7 @@ def install(monkeypatch) -> None:
                  "add_layernorm", "scale_", "head_linear", "latent_write", "latent_attention",
                  "latent_mfma_ok",
                  "sigmoid_gate_", "route", "routed_units", "router_logits", "gelu_tanh",
-                 "depth_mix_", "decay_attention"):
+                 "depth_mix_", "decay_attention", "gelu_erf", "lanes_step", "head_prepare_",
+                 "head_gate_"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

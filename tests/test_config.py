@@ -118,11 +118,11 @@ def test_eos_ids_come_from_generation_config_first(tmp_path):
 
 
 def test_registry_names_the_model_by_its_architecture():
-    assert architecture_names() == ["Bekunex", "Gipotar", "Lagedra", "LlamaForCausalLM"]
+    assert architecture_names() == ["Bekunex", "Gipotar", "Lagedra", "LlamaForCausalLM", "Pamolix"]
     arch = architecture_of(TINY_A)
     spec = arch.build_spec(arch.parse_config(TINY_A))
     assert len(spec.layers) == 2 and spec.vocab_size == 256
-    with pytest.raises(ConfigError, match="MistralForCausalLM.*known: Bekunex, Gipotar, Lagedra, LlamaForCausalLM"):
+    with pytest.raises(ConfigError, match="MistralForCausalLM.*known: Bekunex, Gipotar, Lagedra, LlamaForCausalLM, Pamolix"):
         architecture("MistralForCausalLM")
     with pytest.raises(ConfigError, match="architectures"):
         architecture_of({"hidden_size": 4})
