@@ -1,0 +1,162 @@
+"""Small Pamolix configurations and weights for the tests: sizes that differ from layer to layer
+and between the configurations (one to six heads, grouped and ungrouped key/value heads, key and
+value sizes on either side of each other and off the multiples of 8, whole and partial rotation
+with and without stretched positions, windows of a page, shorter and wider, with no kept first
+keys, a few, a page of them and more than the window; layers with and without the queries'
+factor, layers that read an earlier layer's keys and values, layers without a feed-forward, one
+to four residual streams and none, one expert to all of them chosen, either kind of layer first,
+models of one kind of layer only), and weights at scales at which every mechanism matters: norm
+weights, sinks, biases, gates and the streams' coefficients spread out, scores that reach the
+cap."""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from bekunex_models import judge  # noqa: F401
+from gipotar_models import (as_stored, prompts, row_error, write_folder,  # noqa: F401
+                            TOLERANCE)
+
+
+def _moe(ff, experts, top):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def _dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def _first(heads, kv_heads, dim, vdim, scale, temp, mlp, kv_from=None):
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if temp is not None:
+        mixer["q_temp"] = {"coef": temp[0], "every": temp[1]}
+    if kv_from is not None:
+        mixer["kv_from"] = kv_from
+    return {"type": "attention", "mlp": mlp, "mixer": mixer}
+
+
+def _second(heads, kv_heads, dim, vdim, scale, mask, rot, softcap, mlp):
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if mask is not None:
+        mixer["mask"] = {"keep_first": mask[1], "size": mask[0]}
+    if rot is not None:
+        mixer["rot"] = {"base": rot[1], "dims": rot[0], "scaling": {"factor": rot[2]}}
+    if softcap:
+        mixer["softcap"] = softcap
+    return {"type": "attention_2", "mlp": mlp, "mixer": mixer}
+
+
+# Both kinds of layer; three streams; a layer that reads the first layer's keys and values with
+# another kind between them; windows of 20 with 5 kept, of a page with a page kept, of 33 with
+# none kept; partial and whole rotation; a layer without a feed-forward.
+CONFIG_A = {
+    "architecture": "Pamolix", "vocab": 97, "width": 48, "embedding": {"scale": 1.7},
+    "norm": {"eps": 1e-5}, "streams": 3,
+    "layers": [
+        _first(4, 2, 16, 24, 0.3, (0.4, 16), _dense(72)),
+        _second(6, 2, 8, 12, 0.4, (20, 5), (4, 1000.0, 4.0), 6.0, _moe(24, 6, 2)),
+        _first(4, 2, 16, 24, 0.25, (0.8, 7), None, kv_from=0),
+        _second(2, 2, 24, 12, 0.25, (16, 16), (24, 300.0, 1.0), 9.0, _moe(16, 4, 1)),
+        _first(2, 1, 12, 12, 0.3, None, _moe(20, 8, 4)),
+        _second(3, 1, 12, 20, 0.3, (33, 0), (8, 40000.0, 2.5), 5.0, _dense(40)),
+    ],
+}
+# Only the first kind; one stream (with coefficients); every query head its own key/value head;
+# every expert chosen; sizes off the multiples of 4.
+CONFIG_B = {
+    "architecture": "Pamolix", "vocab": 64, "width": 40, "embedding": {"scale": 0.6},
+    "norm": {"eps": 1e-6}, "streams": 1,
+    "layers": [
+        _first(5, 5, 6, 10, 0.4, (1.5, 3), _moe(12, 3, 3)),
+        _first(1, 1, 70, 33, 0.12, None, None),
+        _first(5, 5, 6, 10, 0.4, (0.2, 40), _dense(56), kv_from=0),
+        _first(2, 1, 30, 16, 0.18, (0.5, 1), _moe(9, 5, 2)),
+    ],
+}
+# Only the second kind; no streams at all (one plain residual sum); a window of one position,
+# more kept keys than the window, no window at all, no rotation at all, no cap; head sizes and
+# rotated widths off the multiples of 8.
+CONFIG_C = {
+    "architecture": "Pamolix", "vocab": 80, "width": 56, "embedding": {"scale": 2.0},
+    "norm": {"eps": 1e-6},
+    "layers": [
+        _second(3, 3, 12, 20, 0.28, (16, 3), (6, 300.0, 1.0), 7.0, _moe(20, 4, 2)),
+        _second(4, 1, 10, 10, 0.3, (1, 2), (10, 1000.0, 3.0), 3.0, None),
+        _second(6, 3, 20, 20, 0.22, (8, 24), None, 0.0, _dense(30)),
+        _second(2, 2, 14, 6, 0.25, None, (4, 20000.0, 16.0), 8.0, _moe(10, 2, 1)),
+    ],
+}
+# Head sizes that the matrix-core kernels take as they are (64 with the whole head rotated, 128
+# and 32 for keys and values, 48 and 64 padded to one size), four streams, for prompts of
+# hundreds of tokens; windows of 100 with 10 kept and of 40 with 70 kept.
+CONFIG_D = {
+    "architecture": "Pamolix", "vocab": 200, "width": 128, "embedding": {"scale": 1.0},
+    "norm": {"eps": 1e-6}, "streams": 4,
+    "layers": [
+        _first(4, 2, 64, 64, 0.125, (0.3, 100), _dense(192)),
+        _second(4, 2, 64, 64, 0.125, (100, 10), (64, 10000.0, 8.0), 15.0, _moe(64, 8, 2)),
+        _first(4, 2, 64, 64, 0.125, (0.6, 64), _moe(32, 4, 3), kv_from=0),
+        _second(2, 1, 128, 32, 0.09, (40, 70), (64, 500000.0, 1.0), 25.0, _dense(160)),
+        _first(4, 1, 48, 64, 0.14, None, None),
+    ],
+}
+# A width, feed-forward widths and a vocabulary that are no multiples of 8 (rows that do not
+# start on 16-byte boundaries in bfloat16), experts of an odd inner width, one head, two streams.
+CONFIG_E = {
+    "architecture": "Pamolix", "vocab": 333, "width": 100, "embedding": {"scale": 3.5},
+    "norm": {"eps": 1e-5}, "streams": 2,
+    "layers": [
+        _second(1, 1, 28, 36, 0.2, (24, 1), (14, 5000.0, 4.0), 12.0, _moe(25, 3, 3)),
+        _first(1, 1, 36, 52, 0.17, (0.3, 10), _dense(150)),
+        _first(3, 1, 20, 36, 0.22, (0.7, 25), _moe(31, 6, 2)),
+        _second(5, 1, 20, 12, 0.22, (60, 7), (20, 900.0, 1.0), 6.0, _dense(70)),
+    ],
+}
+CONFIGS = {"a": CONFIG_A, "b": CONFIG_B, "c": CONFIG_C, "d": CONFIG_D, "e": CONFIG_E}
+
+
+def spec_of(config: dict):
+    from rust_llm_inference_server_amd.registry import architecture_of
+    arch = architecture_of(config)
+    return arch.build_spec(arch.parse_config(config))
+
+
+def make_weights(config: dict, seed: int) -> Dict[str, torch.Tensor]:
+    """float32 tensors by checkpoint name, values chosen by what the tensor is."""
+    g = torch.Generator().manual_seed(seed)
+    normal = lambda shape, std=1.0: torch.randn(shape, generator=g) * std
+    out = {}
+    for t in spec_of(config).tensor_specs():
+        name, shape = t.name, tuple(t.shape)
+        parts = name.split(".")
+        last = parts[-1]
+        if name == "embed":
+            w = normal(shape, 0.5)
+        elif last in ("norm1", "norm2") or name == "final.norm":
+            w = normal(shape, 0.3)                         # stored around zero
+        elif last == "norm":
+            w = 1.0 + normal(shape, 0.3)                   # the heads' norms: plain weights
+        elif last == "sink":
+            w = normal(shape, 1.5)
+        elif last == "b":
+            w = normal(shape, 0.3)
+        elif len(parts) > 2 and parts[1] in ("hc1", "hc2"):
+            if last == "mix":
+                w = torch.eye(shape[0]) + normal(shape, 0.3)
+            else:
+                w = (1.0 if last == "out" else 1.0 / shape[0] + 0.3) + normal(shape, 0.3)
+        elif last == "router":
+            w = normal(shape, 2.0 * shape[1] ** -0.5)
+        elif last == "g":
+            w = normal(shape, 2.0 * shape[1] ** -0.5)
+        elif len(shape) == 2:
+            w = normal(shape, shape[1] ** -0.5)
+        else:
+            raise AssertionError(f"no rule for {name}")
+        out[name] = w.contiguous()
+    return out
+
+
+def plain_logits(plain, cfg: dict, stored: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
+    return plain.forward(cfg, stored, tokens)

@@ -1,0 +1,517 @@
+"""The Pamolix decoder in the engine against the plain implementation (``plain_pamolix.py``):
+whole prompts, token-by-token decoding, portions down to two tokens, batches of unequal
+requests with pages and slots used again, long decoding, keys made to stand out far away, at
+page borders, just inside and just outside every window and every run of kept first keys, a
+sink that outweighs the keys, the first tokens of a sequence, and greedy generation through the
+engine's scheduler.  Every case runs on the GPU (``-m gpu``, float32 and bfloat16) and, with
+the kernels replaced by the slow torch double, on the CPU, where it tests the host logic: the
+run order and whose cache a run reads, the residual streams, windows, the step layout."""
+import copy
+import json
+
+import pytest
+import torch
+
+import pamolix_models as pm
+import plain_pamolix as plain
+import traces
+from rust_llm_inference_server_amd.config import ConfigError, EngineConfig
+from rust_llm_inference_server_amd.sampling import SamplingParams
+
+BACKENDS = ["double", pytest.param("gpu", marks=pytest.mark.gpu)]
+
+
+@pytest.fixture(params=BACKENDS)
+def backend(request):
+    if request.param == "double":
+        import cpu_ops
+        cpu_ops.install(request.getfixturevalue("monkeypatch"))
+        return torch.device("cpu")
+    return torch.device("cuda", 0)
+
+
+@pytest.fixture(params=["float32", pytest.param("bfloat16", marks=pytest.mark.gpu)])
+def dtype(request, backend):
+    if request.param == "bfloat16" and backend.type != "cuda":
+        pytest.skip("bfloat16 runs on the GPU only")
+    return request.param
+
+
+_CACHE = {}
+
+
+def model_case(name, dtype, tmp_path_factory, weights=None, tag="", config=None):
+    """(folder, config, the stored numbers in float64) of a configuration; made once."""
+    key = (name, dtype, tag)
+    if key not in _CACHE:
+        cfg = config if config is not None else pm.CONFIGS[name]
+        w = weights if weights is not None else pm.make_weights(cfg, seed=len(name) + 11)
+        store = torch.float32 if dtype == "float32" else torch.bfloat16
+        folder = pm.write_folder(tmp_path_factory.mktemp(f"pamolix_{name}_{dtype}{tag}"), cfg, w,
+                                 store)
+        _CACHE[key] = (folder, cfg, pm.as_stored(w, store))
+    return _CACHE[key]
+
+
+def runner_for(folder, device, dtype, num_pages=64, page_size=16, max_num_seqs=4,
+               max_positions=512, use_graphs=True):
+    from rust_llm_inference_server_amd.engine import ModelRunner, load_model
+    model = load_model(folder, dtype, max_positions, device)
+    return ModelRunner(model, num_pages=num_pages, page_size=page_size,
+                       max_num_seqs=max_num_seqs, use_graphs=use_graphs)
+
+
+def check_trace(runner, steps, reqs, cfg, stored, dtype):
+    """Replay ``steps`` and hold every wanted row against the plain logits of its request."""
+    outputs = traces.replay_in_process(runner, steps)
+    got = traces.collect(steps, outputs, cfg["vocab"])
+    errors = []
+    for rid, tokens in reqs.items():
+        want = pm.plain_logits(plain, cfg, stored, tokens)
+        assert sorted(got[rid]) == list(range(len(tokens)))
+        errors += [pm.row_error(row, want[pos]) for pos, row in got[rid].items()]
+    pm.judge(errors, dtype)
+
+
+# ----------------------------------------------------------------------- configuration
+def test_config_round_trip_and_the_specification():
+    from rust_llm_inference_server_amd.registry import architecture_of
+    for cfg in pm.CONFIGS.values():
+        arch = architecture_of(cfg)
+        assert arch.name == "Pamolix"
+        assert arch.config_to_dict(arch.parse_config(cfg)) == cfg
+    spec = pm.spec_of(pm.CONFIG_A)
+    names = {t.name: tuple(t.shape) for t in spec.tensor_specs()}
+    assert names["l0.mix.q"] == (64, 48) and names["l0.mix.k"] == (32, 48)
+    assert names["l0.mix.v"] == (48, 48) and names["l0.mix.v.b"] == (48,)
+    assert names["l0.mix.q.norm"] == (16,) and names["l0.mix.sink"] == (4,)
+    assert names["l1.mix.g"] == (6, 48) and "l1.mix.q.b" not in names and "l1.mix.sink" not in names
+    # a layer that reads another's keys and values has none of their tensors
+    assert "l2.mix.q" in names and "l2.mix.q.norm" in names
+    assert not any(n in names for n in ("l2.mix.k", "l2.mix.v", "l2.mix.k.b", "l2.mix.k.norm"))
+    # ... nor a feed-forward, its norm and its connection when it has none
+    assert not any(n.startswith(("l2.mlp", "l2.norm2", "l2.hc2")) for n in names)
+    assert names["l0.hc1.mix"] == (3, 3) and names["l0.hc2.in"] == (3,)
+    assert names["l1.mlp.router.b"] == (6,) and names["l1.mlp.e5.down"] == (48, 24)
+    assert "head" not in names and names["embed"] == (97, 48)
+    runs = spec.runs()
+    assert [r.cache_of for r in runs] == [None, None, 0, None, None, None]
+    # no streams: the plain block, no coefficients
+    plain_names = {t.name for t in pm.spec_of(pm.CONFIG_C).tensor_specs()}
+    assert not any(".hc" in n for n in plain_names)
+    assert pm.spec_of(pm.CONFIG_C).layers[0].block.kind == "prenorm"
+
+
+def _edit(path, value):
+    def apply(cfg):
+        node = cfg
+        for key in path[:-1]:
+            node = node[key]
+        if value is _DROP:
+            del node[path[-1]]
+        else:
+            node[path[-1]] = value
+    return apply
+
+
+_DROP = object()
+
+
+@pytest.mark.parametrize("edit, message", [
+    (_edit(("layers", 0, "type"), "attention_3"), "type 'attention_3'"),
+    (_edit(("layers", 0, "mixer", "kv_heads"), 3), "'kv_heads'"),
+    (_edit(("layers", 1, "mixer", "rot", "dims"), 7), "'dims' 7"),
+    (_edit(("layers", 1, "mixer", "rot", "dims"), 18), "'dims' 18"),
+    (_edit(("layers", 1, "mixer", "rot", "scaling", "factor"), 0.0), "'factor'"),
+    (_edit(("layers", 0, "mixer", "scale"), _DROP), "'scale'"),
+    (_edit(("layers", 0, "mixer", "q_temp", "every"), 0), "'every'"),
+    (_edit(("layers", 1, "mixer", "mask", "keep_first"), -1), "'keep_first'"),
+    (_edit(("layers", 0, "mlp", "kind"), "glu"), "kind 'glu'"),
+    (_edit(("layers", 1, "mlp", "router", "top"), 7), "7 chosen"),
+    (_edit(("layers", 2, "mixer", "kv_from"), 2), "'kv_from' 2"),
+    (_edit(("layers", 2, "mixer", "kv_from"), 1), "'kv_from' 1"),
+    (_edit(("layers", 2, "mixer", "vdim"), 16), "whose keys and values it reads"),
+    (_edit(("norm", "eps"), 0.0), "'eps'"),
+    (_edit(("streams",), 0), "'streams'"),
+    (_edit(("width",), _DROP), "'width'"),
+])
+def test_config_errors_name_the_key(edit, message):
+    from rust_llm_inference_server_amd.registry import architecture_of
+    cfg = copy.deepcopy(pm.CONFIG_A)
+    edit(cfg)
+    with pytest.raises(ConfigError) as e:
+        architecture_of(cfg).parse_config(cfg)
+    assert message in str(e.value)
+
+
+def test_the_plain_implementation_does_not_look_ahead():
+    """A position's plain logits depend on the tokens up to it and on nothing behind it; and
+    they do depend on a token far back (through the layers that see every earlier key)."""
+    cfg = pm.CONFIG_A
+    stored = pm.as_stored(pm.make_weights(cfg, 5), torch.float32)
+    tokens = pm.prompts(cfg["vocab"], [60], seed=1)[0]
+    whole = pm.plain_logits(plain, cfg, stored, tokens)
+    part = pm.plain_logits(plain, cfg, stored, tokens[:41])
+    assert float((whole[:41] - part).abs().max()) < 1e-9
+    other = list(tokens)
+    other[3] = (other[3] + 1) % cfg["vocab"]
+    assert float((pm.plain_logits(plain, cfg, stored, other)[-1] - whole[-1]).abs().max()) > 1e-6
+
+
+# --------------------------------------------------------------------- the step function
+@pytest.mark.parametrize("name", ["a", "b", "c", "e"])
+def test_whole_prompts_and_first_tokens(backend, dtype, name, tmp_path_factory):
+    folder, cfg, stored = model_case(name, dtype, tmp_path_factory)
+    reqs = traces.random_requests(cfg["vocab"], [1, 2, 3, 19, 70], seed=11)
+    steps, _ = traces.trace_whole(reqs)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_decoding_token_by_token_equals_the_prompt_pass(backend, dtype, name, tmp_path_factory):
+    """One request decoded from its first token on, one after a prompt, so that every window
+    passes over decoded tokens and the kept first keys are themselves decoded ones; single
+    tokens go through captured steps on the GPU."""
+    folder, cfg, stored = model_case(name, dtype, tmp_path_factory)
+    reqs = traces.random_requests(cfg["vocab"], [45, 80], seed=12)
+    ids = list(reqs)
+    steps, _ = traces.trace_tail({ids[0]: reqs[ids[0]]}, tail=44)
+    more, _ = traces.trace_tail({ids[1]: reqs[ids[1]]}, tail=45)
+    for s in more:
+        s["step"] += len(steps)
+    check_trace(runner_for(folder, backend, dtype), steps + more, reqs, cfg, stored, dtype)
+
+
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_portions_of_any_size(backend, dtype, name, tmp_path_factory):
+    """Portions of 7, 2, 16, 3, 24, 2, 33, ... tokens: portions that end inside a page, inside
+    a window and inside the kept first keys."""
+    folder, cfg, stored = model_case(name, dtype, tmp_path_factory)
+    reqs = traces.random_requests(cfg["vocab"], [90, 37], seed=13)
+    steps, _ = traces.trace_portions(reqs)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+@pytest.mark.parametrize("name", ["a", "c", "e"])
+def test_mixed_batches_reuse_pages_and_slots(backend, dtype, name, tmp_path_factory):
+    """Seven unequal requests through three slots and a pool that holds three of them: portions
+    beside single tokens, requests left out of steps, pages of finished requests taken by
+    later ones with their old contents still there."""
+    folder, cfg, stored = model_case(name, dtype, tmp_path_factory)
+    reqs = traces.random_requests(cfg["vocab"], [50, 9, 75, 33, 2, 64, 21], seed=14)
+    steps, peak = traces.trace_mixed(reqs, live=3, seed=5)
+    runner = runner_for(folder, backend, dtype, num_pages=-(-peak // 16), max_num_seqs=3)
+    check_trace(runner, steps, reqs, cfg, stored, dtype)
+    assert runner.cache.num_free_pages() == -(-peak // 16)
+
+
+def test_a_request_alone_equals_itself_in_a_batch(backend, dtype, tmp_path_factory):
+    """The rows of a request do not depend on what else the step holds (beyond rounding)."""
+    folder, cfg, stored = model_case("a", dtype, tmp_path_factory)
+    reqs = traces.random_requests(cfg["vocab"], [40, 23, 31], seed=15)
+    alone = {}
+    for rid, tokens in reqs.items():
+        steps, _ = traces.trace_portions({rid: tokens})
+        out = traces.replay_in_process(runner_for(folder, backend, dtype), steps)
+        alone[rid] = traces.collect(steps, out, cfg["vocab"])[rid]
+    steps, _ = traces.trace_mixed(reqs, live=3, seed=2)
+    out = traces.replay_in_process(runner_for(folder, backend, dtype), steps)
+    together = traces.collect(steps, out, cfg["vocab"])
+    pm.judge([pm.row_error(row, alone[rid][pos]) for rid in reqs
+              for pos, row in together[rid].items()], dtype)
+
+
+def test_long_prompts_and_long_decoding(backend, dtype, tmp_path_factory):
+    """A prompt of hundreds of tokens in one step, then hundreds of single-token steps: windows
+    move over many pages while the kept first keys stay, the layers that see everything read
+    ever more partitions, and the queries' factor takes many values."""
+    folder, cfg, stored = model_case("a", dtype, tmp_path_factory)
+    n, tail = (150, 60) if backend.type == "cpu" else (390, 150)
+    reqs = traces.random_requests(cfg["vocab"], [n], seed=16)
+    steps, _ = traces.trace_tail(reqs, tail=tail)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+def test_prompts_of_hundreds_of_tokens_at_head_sizes_of_real_models(backend, dtype,
+                                                                    tmp_path_factory):
+    """Heads of 64 and 128: whole prompts of up to 700 tokens in one step (the attention
+    kernels' tiles of 64 and 128 queries, the rotation inside the attention kernel where the
+    whole head of 64 turns), the same prompts with their ends decoded, and in portions beside
+    each other; at the end a context of more than 1,024 keys, which the decode kernels cut
+    into partitions."""
+    folder, cfg, stored = model_case("d", dtype, tmp_path_factory)
+    lengths = [300, 130] if backend.type == "cpu" else [700, 300, 130, 257]
+    reqs = traces.random_requests(cfg["vocab"], lengths, seed=71)
+    make = lambda: runner_for(folder, backend, dtype, num_pages=130, max_positions=2048)
+    steps, _ = traces.trace_whole(reqs)
+    check_trace(make(), steps, reqs, cfg, stored, dtype)
+    steps, _ = traces.trace_tail(reqs, tail=20)
+    check_trace(make(), steps, reqs, cfg, stored, dtype)
+    steps, peak = traces.trace_mixed(reqs, live=3, seed=6)
+    check_trace(runner_for(folder, backend, dtype, num_pages=-(-peak // 16), max_num_seqs=3,
+                           max_positions=2048), steps, reqs, cfg, stored, dtype)
+    # a long portion beside single decoded tokens of two other requests, in one step
+    reqs = traces.random_requests(cfg["vocab"], [60, 70, 330], seed=72)
+    cuts = [{"r0": (0, 40), "r1": (0, 50)}, {"r0": (40, 41), "r1": (50, 51), "r2": (0, 300)},
+            {"r0": (41, 60), "r1": (51, 70), "r2": (300, 330)}]
+    steps = [{"step": i, "end": [], "entries": [
+        {"id": rid, "tokens": reqs[rid][lo:hi], "want": list(range(hi - lo))}
+        for rid, (lo, hi) in cut.items()]} for i, cut in enumerate(cuts)]
+    steps[-1]["end"] = ["r0", "r1", "r2"]
+    check_trace(make(), steps, reqs, cfg, stored, dtype)
+    if backend.type == "cuda":
+        reqs = traces.random_requests(cfg["vocab"], [1100], seed=73)
+        steps, _ = traces.trace_tail(reqs, tail=40)
+        check_trace(make(), steps, reqs, cfg, stored, dtype)
+
+
+# ------------------------------------------------------------- keys made to stand out
+KEY_TOKEN, QUERY_TOKEN, FILL_TOKEN = 5, 9, 1
+
+
+def _marked(cfg, seed):
+    """Weights in which coordinate 0 of every stream is nonzero at ``KEY_TOKEN`` only and
+    coordinate 1 at ``QUERY_TOKEN`` only, in every layer: the embedding sets them, no layer's
+    output touches them, and the streams' coefficients carry them on as they are.
+    The final norm's weight lets neither through to the tied head."""
+    w = pm.make_weights(cfg, seed=seed)
+    w["final.norm"][:2] = -1.0
+    w["embed"][:, :2] = 0.0
+    w["embed"][KEY_TOKEN, 0] = 3.0
+    w["embed"][QUERY_TOKEN, 1] = 3.0
+    for name, t in w.items():
+        parts = name.split(".")
+        last = parts[-1]
+        if last in ("o", "down"):
+            t[:2] = 0.0
+        elif len(parts) > 2 and parts[1] in ("hc1", "hc2") and last != "out":
+            # the streams' marks stay equal and of one size: what flows into a stream, and what
+            # a sublayer reads, are weighted means
+            t.abs_().clamp_(min=0.2)
+            t /= t.sum(0, keepdim=True)
+        elif last in ("norm1", "norm2"):
+            t.clamp_(min=-0.5)
+    return w
+
+
+def _attention_stands_out(cfg, w, layer, boost=8.0):
+    """In every head of ``layer``'s attention the key of ``KEY_TOKEN`` gets a score far above
+    the others' from a query of ``QUERY_TOKEN``: one channel of every key head reads stream
+    coordinate 0, the same channel of every query head coordinate 1.  In a layer that rotates,
+    the channel is one that is not rotated, or else the slowest rotated pair's first half (whose
+    partner is emptied); in a layer that normalises its heads, the heads' norm weights let that
+    channel through at twice its size and the biases leave it alone."""
+    m = cfg["layers"][layer]["mixer"]
+    p = f"l{layer}.mix"
+    d = m["dim"]
+    dims = (m.get("rot") or {}).get("dims", 0)
+    chans = [dims] if dims < d else [dims // 2 - 1, dims - 1]
+    source = p if m.get("kv_from") is None else f"l{m['kv_from']}.mix"
+    for name, heads, where in (("q", m["heads"], p), ("k", m["kv_heads"], source)):
+        for head in range(heads):
+            for n, c in enumerate(chans):
+                row = head * d + c
+                w[f"{where}.{name}"][row] = 0.0
+                if n == 0:
+                    w[f"{where}.{name}"][row, 1 if name == "q" else 0] = boost
+                if f"{where}.{name}.b" in w:
+                    w[f"{where}.{name}.b"][row] = 0.0
+        if f"{where}.{name}.norm" in w:
+            w[f"{where}.{name}.norm"][chans[0]] = 2.0
+    if "softcap" in m:
+        m["softcap"] = max(m["softcap"], 12.0)   # far above what hundreds of other keys add up to
+    if f"{p}.sink" in w:
+        w[f"{p}.sink"].clamp_(max=1.0)
+    return w
+
+
+def _tokens(vocab, n, seed):
+    return [t if t not in (KEY_TOKEN, QUERY_TOKEN) else FILL_TOKEN
+            for t in pm.prompts(vocab, [n], seed=seed)[0]]
+
+
+@pytest.mark.parametrize("layer, back", [(1, 19), (1, 20), (3, 15), (3, 16), (5, 32), (5, 33)])
+def test_keys_just_inside_and_outside_every_window(backend, dtype, layer, back,
+                                                   tmp_path_factory):
+    """Windows of 20, 16 (a page) and 33 positions.  A key that stands out lies ``back``
+    positions behind the query: the last one inside or the first one outside (and beyond the
+    kept first keys).  A window that is one token off, in a prompt's portion or decoded alone,
+    moves the row far."""
+    cfg = copy.deepcopy(pm.CONFIG_A)
+    size = cfg["layers"][layer]["mixer"]["mask"]["size"]
+    w = _attention_stands_out(cfg, _marked(cfg, seed=31 + layer), layer)
+    folder, _, stored = model_case("a", dtype, tmp_path_factory, weights=w,
+                                   tag=f"edge{layer}", config=cfg)
+    n = back + 70
+    tokens = _tokens(cfg["vocab"], n, seed=32)
+    queries = (back + 25, n - 4)                 # one in the prompt's part, one decoded
+    for query in queries:
+        tokens[query] = QUERY_TOKEN
+        tokens[query - back] = KEY_TOKEN
+    other = copy.deepcopy(cfg)
+    other["layers"][layer]["mixer"]["mask"]["size"] += -1 if back == size - 1 else 1
+    a, b = pm.plain_logits(plain, cfg, stored, tokens), pm.plain_logits(plain, other, stored, tokens)
+    for query in queries:
+        assert pm.row_error(a[query], b[query]) > 0.03
+    reqs = {"r": tokens}
+    steps, _ = traces.trace_tail(reqs, tail=12)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+    steps, _ = traces.trace_portions(reqs)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+@pytest.mark.parametrize("layer, at", [(1, 4), (1, 5), (3, 15), (3, 16)])
+def test_the_last_kept_first_key_and_the_one_behind_it(backend, dtype, layer, at,
+                                                       tmp_path_factory):
+    """5 and 16 (a page of) kept first keys.  The key that stands out lies at position ``at``:
+    the last kept one or the first that is not, far in front of every window that the queries
+    (in the prompt's part and decoded) have.  A count of kept keys that is one off moves the
+    rows far."""
+    cfg = copy.deepcopy(pm.CONFIG_A)
+    keep = cfg["layers"][layer]["mixer"]["mask"]["keep_first"]
+    w = _attention_stands_out(cfg, _marked(cfg, seed=51 + layer), layer)
+    folder, _, stored = model_case("a", dtype, tmp_path_factory, weights=w,
+                                   tag=f"kept{layer}", config=cfg)
+    tokens = _tokens(cfg["vocab"], 120, seed=52)
+    tokens[at] = KEY_TOKEN
+    queries = (70, 116)
+    for query in queries:
+        tokens[query] = QUERY_TOKEN
+    other = copy.deepcopy(cfg)
+    other["layers"][layer]["mixer"]["mask"]["keep_first"] += -1 if at == keep - 1 else 1
+    a, b = pm.plain_logits(plain, cfg, stored, tokens), pm.plain_logits(plain, other, stored, tokens)
+    for query in queries:
+        assert pm.row_error(a[query], b[query]) > 0.03
+    reqs = {"r": tokens}
+    steps, _ = traces.trace_tail(reqs, tail=12)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+    steps, _ = traces.trace_portions(reqs)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+@pytest.mark.parametrize("layer", [0, 2])
+@pytest.mark.parametrize("far", [0, 15, 16, 17, 48])
+def test_a_far_key_that_stands_out(backend, dtype, layer, far, tmp_path_factory):
+    """Layers that see every earlier key, over pages of 16 (one of them through the keys that
+    another layer cached): the token at ``far`` (a page's first or last position among them)
+    takes most of the weight of queries 140 and more positions on, in a prompt's portion and
+    decoded alone.  Were its row lost or read from a wrong page, the layer would return another
+    token's value."""
+    cfg = copy.deepcopy(pm.CONFIG_A)
+    w = _attention_stands_out(cfg, _marked(cfg, seed=41), layer)
+    folder, _, stored = model_case("a", dtype, tmp_path_factory, weights=w, tag=f"far{layer}",
+                                   config=cfg)
+    tokens = _tokens(cfg["vocab"], 200, seed=42)
+    tokens[far] = KEY_TOKEN
+    tokens[far + 140] = tokens[197] = QUERY_TOKEN
+    moved = list(tokens)
+    moved[far] = FILL_TOKEN
+    a, b = pm.plain_logits(plain, cfg, stored, tokens), pm.plain_logits(plain, cfg, stored, moved)
+    assert pm.row_error(a[far + 140], b[far + 140]) > 0.03 and pm.row_error(a[197], b[197]) > 0.03
+    reqs = {"r": tokens}
+    steps, _ = traces.trace_tail(reqs, tail=6)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+def test_a_sink_that_outweighs_the_keys(backend, dtype, tmp_path_factory):
+    """Sinks of 4 and more in a model of sink layers only: most of every row's weight goes to
+    no value at all.  Left out, or counted per key, the rows move far; and a sink far below the
+    scores changes nothing."""
+    cfg = pm.CONFIG_B
+    w = pm.make_weights(cfg, seed=61)
+    for name in w:
+        if name.endswith(".sink"):
+            w[name] = w[name].abs() + 4.0
+    w["l1.mix.sink"][:] = -30.0
+    folder, _, stored = model_case("b", dtype, tmp_path_factory, weights=w, tag="sink")
+    tokens = pm.prompts(cfg["vocab"], [50], seed=62)[0]
+    without = {k: (v - 40.0 if k.endswith(".sink") else v) for k, v in stored.items()}
+    a, b = pm.plain_logits(plain, cfg, stored, tokens), pm.plain_logits(plain, cfg, without, tokens)
+    assert min(pm.row_error(a[i], b[i]) for i in range(50)) > 0.03
+    reqs = {"r": tokens}
+    steps, _ = traces.trace_tail(reqs, tail=20)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+    steps, _ = traces.trace_portions(reqs)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+def test_scores_reach_the_cap(backend, dtype, tmp_path_factory):
+    """Query and key projections ten times as large: most scores of the capped layers sit at
+    the cap, where it, not the product, decides the weights."""
+    cfg = pm.CONFIG_C
+    w = pm.make_weights(cfg, seed=81)
+    for i, layer in enumerate(cfg["layers"]):
+        if layer["mixer"].get("softcap"):
+            w[f"l{i}.mix.q"] *= 10.0
+    folder, _, stored = model_case("c", dtype, tmp_path_factory, weights=w, tag="cap")
+    reqs = traces.random_requests(cfg["vocab"], [40, 24], seed=82)
+    steps, _ = traces.trace_tail(reqs, tail=10)
+    check_trace(runner_for(folder, backend, dtype), steps, reqs, cfg, stored, dtype)
+
+
+# -------------------------------------------------------------------- engine and scheduler
+def test_greedy_generation_through_the_engine(backend, dtype, tmp_path_factory):
+    """Five requests through three seats with a token budget that cuts the prompts: every
+    generated token is the plain implementation's pick, up to a near-tie of its logits."""
+    from rust_llm_inference_server_amd.engine import Engine, load_model
+    folder, cfg, stored = model_case("a", dtype, tmp_path_factory)
+    model = load_model(folder, dtype, 256, backend)
+    engine = Engine(model, EngineConfig(max_num_seqs=3, max_batched_tokens=16, num_pages=48,
+                                        block_size=8, max_seq_len=256, watermark_pages=1))
+    prompts = pm.prompts(cfg["vocab"], [5, 21, 1, 34, 12], seed=18)
+    outs = engine.generate(prompts, SamplingParams.greedy(7))
+    margin = 1e-3 if dtype == "float32" else 0.5
+    for p, o in zip(prompts, outs):
+        assert o.finish_reason == "length" and len(o.token_ids) == 7
+        tokens = list(p)
+        for got in o.token_ids:
+            last = pm.plain_logits(plain, cfg, stored, tokens)[-1]
+            best = int(torch.argmax(last))
+            if got != best:
+                assert float(last[best] - last[got]) < margin
+            tokens.append(got)
+    engine.runner.cache.check_invariants()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_the_replay_program_runs_the_model(dtype_name, tmp_path_factory, tmp_path):
+    folder, cfg, stored = model_case("a", dtype_name, tmp_path_factory)
+    reqs = traces.random_requests(cfg["vocab"], [40, 7, 25, 33, 18], seed=19)
+    steps, peak = traces.trace_mixed(reqs, live=4, seed=3)
+    out = traces.replay_program(folder, dtype_name, steps, peak, str(tmp_path / "out"),
+                                cfg["vocab"])
+    got = traces.collect(steps, out, cfg["vocab"])
+    errors = []
+    for rid, tokens in reqs.items():
+        want = pm.plain_logits(plain, cfg, stored, tokens)
+        errors += [pm.row_error(row, want[pos]) for pos, row in got[rid].items()]
+    pm.judge(errors, dtype_name)
+
+
+@pytest.mark.gpu
+def test_the_command_line_generates_and_scores(tmp_path_factory, tmp_path, capsys):
+    """``rlis generate`` picks the design by config.json and prints the plain implementation's
+    greedy tokens; ``rlis perplexity`` scores a token file through the same step function."""
+    from rust_llm_inference_server_amd import cli
+    folder, cfg, stored = model_case("b", "float32", tmp_path_factory)
+    prompt = pm.prompts(cfg["vocab"], [11], seed=20)[0]
+    rc = cli.main(["generate", "--model", folder, "--dtype", "f32", "--max-seq-len", "128",
+                   "--num-pages", "32", "--block-size", "8", "--max-num-seqs", "2",
+                   "--max-tokens", "5", "--prompt-ids", ",".join(map(str, prompt))])
+    out = capsys.readouterr()
+    assert rc == 0
+    got = [int(t) for t in out.out.split()]
+    tokens = list(prompt)
+    for g in got:
+        last = pm.plain_logits(plain, cfg, stored, tokens)[-1]
+        best = int(torch.argmax(last))
+        assert g == best or float(last[best] - last[g]) < 1e-3
+        tokens.append(g)
+    assert len(got) == 5 and "output 5 tok (length)" in out.err
+    ids = tmp_path / "ids.txt"
+    ids.write_text(" ".join(map(str, pm.prompts(cfg["vocab"], [96], seed=21)[0])))
+    rc = cli.main(["perplexity", "--model", folder, "--dtype", "f32", "--max-seq-len", "128",
+                   "--ids-file", str(ids), "--ctx", "32"])
+    out = capsys.readouterr()
+    assert rc == 0 and json.loads(out.out.strip().splitlines()[-1])["ppl"] > 1.0
