@@ -10,7 +10,8 @@ typedef int (*PrefillUnit)(const void* q, long long q_stride, void* out, long lo
                            int page_shift, int window, float scale, int tile_queries, int splits,
                            int row0, float* part_ml, float* part_acc, const float* cos,
                            const float* sin, int rot, const float* slopes,
-                           const float* head_scales, float softcap, hipStream_t stream);
+                           const float* head_scales, float softcap, const float* sinks,
+                           int keep_first, hipStream_t stream);
 typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long long out_stride,
                           float* part_ml, float* part_acc, const void* k_pages,
                           const void* v_pages, const int* block_tables, int max_pages,
@@ -18,7 +19,8 @@ typedef int (*DecodeUnit)(const void* q, long long q_stride, void* out, long lon
                           int window, float scale, int splits, int part_keys, int max_parts,
                           int merge_inside, int groups, int cap, const DecodeRope* rope,
                           const DecodeMerge* merge, const float* slopes,
-                          const float* head_scales, float softcap, hipStream_t stream);
+                          const float* head_scales, float softcap, const float* sinks,
+                          int keep_first, hipStream_t stream);
 
 // The units (attention_mfma.hip compiled for a padded head size of 32, 64, ... 256) are
 // libraries of their own, built and loaded when a model needs them and registered here.
@@ -76,7 +78,9 @@ int rlis_launch_attn_reduce_bf16(void* out, long long out_stride, const float* p
 // slopes != null: nh float32 values, one per query head; slopes[head] * (key position - query
 // position) is added to every score in float32 before the softmax.  head_scales != null: nh
 // float32 values that multiply their head's score scale; softcap c > 0: the scaled score becomes
-// c * tanh(score / c) in front of the bias.
+// c * tanh(score / c) in front of the bias.  sinks != null: nh float32 values; e^sink of the head
+// joins every row's denominator once, with no key and no value.  keep_first n > 0 (with a
+// window): the sequence's first n keys stay visible to every later query beside the window's.
 RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out,
                                     long long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_tables, int max_pages,
@@ -86,7 +90,8 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
                                     int splits, int row0, float* part_ml,
                                     float* part_acc, const float* cos, const float* sin,
                                     int rot, const float* slopes, const float* head_scales,
-                                    float softcap, hipStream_t stream) {
+                                    float softcap, const float* sinks, int keep_first,
+                                    hipStream_t stream) {
   // unit_map lists tiles of tile_queries new tokens: 64 (0 means that too) or 128.
   if (tile_queries == 0) tile_queries = 64;
   RLIS_REQUIRE(tile_queries == 64 || tile_queries == 128,
@@ -97,6 +102,7 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
   RLIS_REQUIRE(splits == 1 || (part_ml && part_acc && row0 >= 0 && d % 4 == 0),
                "attn_prefill_mfma: key runs need a workspace and the first row they cover");
   RLIS_REQUIRE(scale > 0.f, "attn_prefill_mfma: the score scale must be positive, got %g", scale);
+  RLIS_REQUIRE(keep_first >= 0, "attn_prefill_mfma: bad count of kept first keys");
   RLIS_REQUIRE(nh % nkv == 0, "attn_prefill_mfma: %d query heads are not a multiple of %d KV heads",
                nh, nkv);
   RLIS_REQUIRE(d % 16 == 0 && d <= 256,
@@ -116,7 +122,8 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
       "attn_prefill_mfma",
       unit(q, q_stride, out, out_stride, k_pages, v_pages, block_tables, max_pages, cu_seqlens,
            start_pos, unit_map, num_tiles, nh, nkv, d, page_shift, window, scale, tile_queries,
-           splits, row0, part_ml, part_acc, cos, sin, rot, slopes, head_scales, softcap, stream),
+           splits, row0, part_ml, part_acc, cos, sin, rot, slopes, head_scales, softcap, sinks,
+           keep_first, stream),
       d);
 }
 
@@ -146,8 +153,8 @@ RLIS_API int rlis_attn_prefill_mfma(const void* q, long long q_stride, void* out
 // whoever computes them; fewer workgroups pay fewer start-ups and hand-overs, which a batch
 // that fills the chip anyway does not need.
 //
-// slopes, head_scales and softcap as in rlis_attn_prefill_mfma (the query's position is the last
-// of its context).
+// slopes, head_scales, softcap, sinks and keep_first as in rlis_attn_prefill_mfma (the query's
+// position is the last of its context).
 RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    long long out_stride, float* part_ml, float* part_acc,
                                    void* k_pages, void* v_pages,
@@ -158,8 +165,8 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                                    const float* cos, const float* sin,
                                    int rot, const int* positions, const int* slots,
                                    long long k_off, long long v_off, const float* slopes,
-                                   const float* head_scales, float softcap,
-                                   hipStream_t stream) {
+                                   const float* head_scales, float softcap, const float* sinks,
+                                   int keep_first, hipStream_t stream) {
   DecodeRope rope;
   rope.cos = positions ? cos : nullptr;
   rope.sin = positions ? sin : nullptr;
@@ -178,6 +185,7 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
                v_off, q_stride);
   RLIS_REQUIRE(S >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0, "attn_decode_mfma: bad sizes");
   RLIS_REQUIRE(scale > 0.f, "attn_decode_mfma: the score scale must be positive, got %g", scale);
+  RLIS_REQUIRE(keep_first >= 0, "attn_decode_mfma: bad count of kept first keys");
   RLIS_REQUIRE(nh % nkv == 0 && nh / nkv <= 16,
                "attn_decode_mfma: %d query heads per KV head, at most 16", nkv ? nh / nkv : 0);
   RLIS_REQUIRE(d % 16 == 0 && d <= 256,
@@ -212,11 +220,12 @@ RLIS_API int rlis_attn_decode_mfma(const void* q, long long q_stride, void* out,
       "attn_decode_mfma",
       unit(q, q_stride, out, out_stride, part_ml, part_acc, k_pages, v_pages, block_tables,
            max_pages, ctx_lens, S, nh, nkv, d, page_shift, window, scale, splits, part_keys,
-           max_parts, inside, groups, cap, &rope, &merge, slopes, head_scales, softcap, stream),
+           max_parts, inside, groups, cap, &rope, &merge, slopes, head_scales, softcap, sinks,
+           keep_first, stream),
       d);
   if (rc) return rc;
   if (splits > 1 && S > 0 && !inside)
-    return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, nullptr,
+    return rlis_launch_attn_reduce_bf16(out, out_stride, part_ml, part_acc, S, nh, d, splits, sinks,
                                         stream);
   return 0;
 }

@@ -118,7 +118,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     int page_shift, float scale, int window, int num_tiles, int tiles_per_round, int part_stride,
     int row0, float* __restrict__ part_ml, float* __restrict__ part_acc,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    const float* __restrict__ slopes, const float* __restrict__ head_scales, float softcap) {
+    const float* __restrict__ slopes, const float* __restrict__ head_scales, float softcap,
+    const float* __restrict__ sinks, int keep_first) {
   constexpr int BN = tile_keys(QB);
   // V^T tile rows: 64 keys padded to a stride of 32 bytes mod 64; 32 keys unpadded, with the
   // 16-byte piece index XORed with (-(row / 4)) & 3, which frees reads and stores of conflicts.
@@ -211,12 +212,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   const int khi_all = P + q_last + 1;                    // keys [klo, khi_all) matter to the tile
   int klo = 0;
   if (window > 0) klo = max(0, P + qb - window + 1);
-  const int kt0_all = (klo / BN) * BN;
-  int kt0 = kt0_all, khi = khi_all;                      // this workgroup's run of them
+  int kt0_all = (klo / BN) * BN;
+  // With first keys of the sequence that stay visible in front of the window, the tile walks
+  // two runs of key tiles: those that hold kept keys, [0, kept_end), and the window's from
+  // kt0_all on.  The walk below runs over one gapless range of *walk positions*: a walk
+  // position x is key x up to kept_end and key x + gap beyond (RLIS_KEY_AT); both are
+  // multiples of the tile size.  Without kept keys, or where the two runs touch, gap is 0.
+  int kept_end = 0, gap = 0;
+  if (window > 0 && keep_first > 0 && kt0_all > 0) {
+    kept_end = ((min(keep_first, klo) + BN - 1) / BN) * BN;
+    if (kept_end >= kt0_all) {
+      kept_end = 0;
+      kt0_all = 0;
+    } else {
+      gap = kt0_all - kept_end;
+      kt0_all = 0;
+    }
+  }
+#define RLIS_KEY_AT(x_) ((x_) < kept_end ? (x_) : (x_) + gap)
+  const int khi_walk = khi_all - gap;
+  int kt0 = kt0_all, khi = khi_walk;                     // this workgroup's run of them
   if (splits > 1) {
-    const int per = ((khi_all - kt0_all + BN - 1) / BN + splits - 1) / splits;
+    const int per = ((khi_walk - kt0_all + BN - 1) / BN + splits - 1) / splits;
     kt0 = kt0_all + split * per * BN;
-    khi = min(khi_all, kt0 + per * BN);
+    khi = min(khi_walk, kt0 + per * BN);
   }
   const int wave_q_last = min(n_new - 1, wave_q_first + 16 * QB - 1);
 
@@ -252,7 +271,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   // larger than tiles: what changes from tile to tile is uniform over the workgroup.  The page
   // index is clamped to the last page of the range; 64 bits are needed only for page id times
   // the elements of a page.
-  const int last_page = (khi - 1) >> page_shift;
+  const int last_page = RLIS_KEY_AT(khi - 1) >> page_shift;
   const unsigned page_elems = ((unsigned)nkv << page_shift) * (unsigned)d;
   int k_pg[KCH], v_pg[VCH];
   unsigned k_in[KCH], v_in[VCH];
@@ -313,15 +332,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   const float inv_cap = (BIAS && softcap > 0.f) ? 1.0f / softcap : 0.f;
   const float in_exp = BIAS ? 1.f : scale2;
   if (kt0 < khi) {           // else this run has no keys (only with splits)
-  RLIS_LOAD_PAGES(kt0, page_ka, page_va);
-  RLIS_LOAD_PAGES(kt0 + BN, page_kb, page_vb);
-  RLIS_LOAD_TILE(kt0, page_ka, page_va, tile_ka, tile_va);
-  RLIS_LOAD_TILE(kt0 + BN, page_kb, page_vb, tile_kb, tile_vb);
-  RLIS_LOAD_PAGES(kt0 + 2 * BN, page_ka, page_va);
-  RLIS_LOAD_PAGES(kt0 + 3 * BN, page_kb, page_vb);
+  RLIS_LOAD_PAGES(RLIS_KEY_AT(kt0), page_ka, page_va);
+  RLIS_LOAD_PAGES(RLIS_KEY_AT(kt0 + BN), page_kb, page_vb);
+  RLIS_LOAD_TILE(RLIS_KEY_AT(kt0), page_ka, page_va, tile_ka, tile_va);
+  RLIS_LOAD_TILE(RLIS_KEY_AT(kt0 + BN), page_kb, page_vb, tile_kb, tile_vb);
+  RLIS_LOAD_PAGES(RLIS_KEY_AT(kt0 + 2 * BN), page_ka, page_va);
+  RLIS_LOAD_PAGES(RLIS_KEY_AT(kt0 + 3 * BN), page_kb, page_vb);
   RLIS_STORE_TILE(tile_ka, tile_va, 0);
-  RLIS_LOAD_TILE(kt0 + 2 * BN, page_ka, page_va, tile_ka, tile_va);
-  RLIS_LOAD_PAGES(kt0 + 4 * BN, page_ka, page_va);
+  RLIS_LOAD_TILE(RLIS_KEY_AT(kt0 + 2 * BN), page_ka, page_va, tile_ka, tile_va);
+  RLIS_LOAD_PAGES(RLIS_KEY_AT(kt0 + 4 * BN), page_ka, page_va);
   // The unrotated queries are turned by the angles asked for above (rotate-half over the
   // whole head): dim j of a lane's fragment ks meets dim j + D / 2 in its fragment ks + D / 64.
   // Here, behind the first tiles' loads, nothing is waited for that has not arrived anyway.
@@ -383,7 +402,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
       }
       // ---- scale, mask (only where a tile meets the diagonal, the window or the end) -----
       const bool plain_tile = (k0 + BN - 1 <= P + wave_q_first) &&
-                              (window <= 0 || k0 > P + wave_q_first + 16 * QB - 1 - window);
+                              (window <= 0 || k0 > P + wave_q_first + 16 * QB - 1 - window ||
+                               k0 + BN <= keep_first);
       // The scale (positive) is applied inside the exponent, with one fused multiply-add per
       // score; the maximum is taken over the raw scores and scaled once.
       bool moved = false;
@@ -402,7 +422,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const int kpos = k0 + (nb / 2) * 32 + lq * 8 + 2 * r + (nb % 2);
-              const bool ok = (kpos <= my_qpos[b]) && (window <= 0 || kpos > my_qpos[b] - window);
+              const bool ok = (kpos <= my_qpos[b]) &&
+                              (window <= 0 || kpos > my_qpos[b] - window || kpos < keep_first);
               const float sv = ok ? s[b][nb][r] : -INFINITY;
               s[b][nb][r] = sv;
               mx = fmaxf(mx, sv);
@@ -470,19 +491,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
   {                                                   \
     if (kTileBufs == 2) {                             \
       if ((k0_) + BN < khi) RLIS_STORE_TILE(TK, TV, 1 - (cur_)); \
-      RLIS_LOAD_TILE((k0_) + 3 * BN, PK, PV, TK, TV); \
-      RLIS_LOAD_PAGES((k0_) + 5 * BN, PK, PV);        \
-      compute(k0_, cur_);                             \
+      RLIS_LOAD_TILE(RLIS_KEY_AT((k0_) + 3 * BN), PK, PV, TK, TV); \
+      RLIS_LOAD_PAGES(RLIS_KEY_AT((k0_) + 5 * BN), PK, PV);        \
+      compute(RLIS_KEY_AT(k0_), cur_);                \
       __syncthreads();                                \
     } else {                                          \
-      compute(k0_, 0);                                \
+      compute(RLIS_KEY_AT(k0_), 0);                   \
       __syncthreads();                                \
       if ((k0_) + BN < khi) {                         \
         RLIS_STORE_TILE(TK, TV, 0);                   \
         __syncthreads();                              \
       }                                               \
-      RLIS_LOAD_TILE((k0_) + 3 * BN, PK, PV, TK, TV); \
-      RLIS_LOAD_PAGES((k0_) + 5 * BN, PK, PV);        \
+      RLIS_LOAD_TILE(RLIS_KEY_AT((k0_) + 3 * BN), PK, PV, TK, TV); \
+      RLIS_LOAD_PAGES(RLIS_KEY_AT((k0_) + 5 * BN), PK, PV);        \
     }                                                 \
   }
   for (int k0 = kt0; k0 < khi; k0 += 2 * BN) {
@@ -494,6 +515,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
 #undef RLIS_LOAD_TILE
 #undef RLIS_LOAD_PAGES
   }
+#undef RLIS_KEY_AT
 
   // ---- normalise and store: this lane holds dims db * 16 + lq * 4 + [0, 4) of its queries --
 #pragma unroll
@@ -503,6 +525,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((QB == 1 &&
     if (my_qi[b] < n_new) {
       const long long row = tok_begin + my_qi[b];
       if (splits == 1) {
+        if (sinks) {
+          // e^sink joins the denominator once (the maxima are base-2 exponents)
+          const float sink2 = sinks[h] * 1.4426950408889634f;
+          const float m_new = fmaxf(m_run[b], sink2);
+          const float corr = __builtin_amdgcn_exp2f(m_run[b] - m_new);
+          l_run[b] = l_run[b] * corr + __builtin_amdgcn_exp2f(sink2 - m_new);
+#pragma unroll
+          for (int db = 0; db < D / 16; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o_acc[b][db][r] *= corr;
+        }
         const float inv_l = 1.0f / l_run[b];
         bf16_t* orow = out + row * out_stride + h * d;
 #pragma unroll
@@ -546,7 +579,8 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
     const int* start_pos, const int* tile_map, int num_tiles, int nh, int nkv, int d,
     int page_shift, int window, float scale, int tile_queries, int splits, int row0,
     float* part_ml, float* part_acc, const float* cos, const float* sin, int rot,
-    const float* slopes, const float* head_scales, float softcap, hipStream_t stream) {
+    const float* slopes, const float* head_scales, float softcap, const float* sinks,
+    int keep_first, hipStream_t stream) {
   if (num_tiles == 0) return 0;
   const bool shaped = slopes || head_scales || softcap > 0.f;
   // rotation inside the kernel needs head_dim = rotated width = 64, 128 or 256
@@ -560,7 +594,7 @@ RLIS_API int RLIS_CAT(rlis_attn_prefill_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages,              \
       (const bf16_t*)v_pages, block_tables, max_pages, cu_seqlens, start_pos, tile_map, nh, nkv, \
       d, page_shift, scale, window, num_tiles, tiles_per_round, splits, row0, part_ml, part_acc, \
-      cos, sin, slopes, head_scales, softcap)
+      cos, sin, slopes, head_scales, softcap, sinks, keep_first)
   if (tile_queries == 2 * BM) {
     if (shaped) RLIS_PREFILL_LAUNCH(2, true);
     else RLIS_PREFILL_LAUNCH(2, false);
@@ -666,11 +700,13 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     int nh, int nkv, int d, int page_shift, float scale, int window, int splits, int part_keys,
     int max_parts, int merge_inside, int groups, int cap, const DecodeRope rope,
     const DecodeMerge merge, const float* __restrict__ slopes,
-    const float* __restrict__ head_scales, float softcap) {
+    const float* __restrict__ head_scales, float softcap, const float* __restrict__ sinks,
+    int keep_first) {
   if constexpr (EXACT) {
     d = D;
     page_shift = kExactPageShift;
     window = 0;
+    keep_first = 0;
   }
   // per partition that the workgroup walks: ml waves * g * 2, then acc waves * g * d
   extern __shared__ float dsm[];
@@ -714,12 +750,30 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   const int* table = block_tables + (long long)seq * max_pages;
   const int page_mask = (1 << page_shift) - 1;
   const int lo = (window > 0 && ctx - window > 0) ? ctx - window : 0;
-  const int lo32 = lo & ~31;
+  int lo32 = lo & ~31;
+  // With first keys of the sequence that stay visible in front of the window, the keys walked
+  // are two runs: the chunks that hold kept keys, [0, kept32), and the window's from lo32 on.
+  // Partitions are laid over one gapless range of *walk positions*: walk position x is key x up
+  // to kept32 and key x + gap beyond (RLIS_KEY_AT); both are multiples of a chunk.  Without
+  // kept keys, or where the two runs touch, gap is 0.  `end` is the context's end as a walk
+  // position.
+  int kept32 = 0, gap = 0;
+  if (!EXACT && keep_first > 0 && lo32 > 0) {
+    kept32 = (min(keep_first, lo) + 31) & ~31;
+    if (kept32 >= lo32) {
+      kept32 = 0;
+    } else {
+      gap = lo32 - kept32;
+    }
+    lo32 = 0;
+  }
+#define RLIS_KEY_AT(x_) ((x_) < kept32 ? (x_) : (x_) + gap)
+  const int end = ctx - gap;
   constexpr int kStride = 32 * kDecodeWaves;       // keys between two chunks of one wave
-  const int part = decode_part_len(ctx - lo32, part_keys, max_parts);   // a multiple of kStride
+  const int part = decode_part_len(end - lo32, part_keys, max_parts);   // a multiple of kStride
   // Merging inside: only the partitions that hold keys of this sequence run, and the last of
   // them to finish merges them all; a sequence with one such partition stores its result itself.
-  const int own = merge_inside ? max(1, min(splits, (ctx - lo32 + part - 1) / part)) : splits;
+  const int own = merge_inside ? max(1, min(splits, (end - lo32 + part - 1) / part)) : splits;
   // This workgroup's partitions: first .. first + mine, one of `sharers` even shares.
   int sharers = own, first = split, mine = 1;
   if constexpr (WALKS) {
@@ -729,7 +783,8 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   }
   if (split >= sharers) return;
   const int kbeg = lo32 + first * part;
-  const int kend = min(ctx, kbeg + mine * part);
+  const int kend = min(end, kbeg + mine * part);
+  const int kend_key = RLIS_KEY_AT(max(kend - 1, 0)) + 1;    // the key behind the last one walked
 
   // A wave takes its chunks two at a time: the page ids of both, then all their keys and
   // values, are on their way before the first product, and the page ids of the next two follow
@@ -738,7 +793,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   // probability exactly zero; values past the end inside a group of 4 keys are whatever the
   // page holds, and the pages only ever hold zeros or values that a model wrote); a dim past d
   // reads one below d (it meets a zero of q, or a row of O^T that is not stored).
-  const int last_key = max(kend - 1, 0), last_quad = last_key & ~3;
+  const int last_key = max(kend_key - 1, 0), last_quad = last_key & ~3;
   int k_dim[D / 32], v_dim[D / 16];
 #pragma unroll
   for (int ks = 0; ks < D / 32; ++ks) k_dim[ks] = min(ks * 32 + lq * 8, d - 8);
@@ -781,10 +836,10 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   int c0 = kbeg + wave * 32;
   constexpr bool kPairs = D <= 128;      // wider heads have no registers for two chunks
   const bool one_by_one = part <= kStride || !kPairs;
-  RLIS_DEC_PAGES(c0, pk_a, pv_a);
+  RLIS_DEC_PAGES(RLIS_KEY_AT(c0), pk_a, pv_a);
   if constexpr (kPairs) {
     // (clamped loads: harmless where a wave has one chunk only, and no branch around loads)
-    RLIS_DEC_PAGES(c0 + kStride, pk_b, pv_b);
+    RLIS_DEC_PAGES(RLIS_KEY_AT(c0 + kStride), pk_b, pv_b);
   }
   // The angles, again without a branch: where nothing is rotated the q row itself (D / 2
   // floats are D bf16 elements of it) is read instead and dropped.
@@ -808,7 +863,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   const float k_cos = k_turns ? k_cos_read : 1.f, k_sin = k_turns ? k_sin_read : 0.f;
 
   // ---- the step's own key and value go to the pages before anyone reads them back --------
-  if (stores_kv && kbeg < ctx && kend == ctx) {
+  if (stores_kv && kbeg < end && kend == end) {
     // This workgroup's partition ends with the step's own key.
     if (slot >= 0 && kv_thread) {
       const long long page = slot >> page_shift;
@@ -869,7 +924,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
         if constexpr (BIAS)
           s[nb][r] = shaped_score(s[nb][r], shaped, softcap, inv_cap,
                                   slope2 * (float)(key - (ctx - 1)));
-        const float sv = (key >= lo && key < kend) ? s[nb][r] : -INFINITY;
+        const float sv = ((key >= lo || key < keep_first) && key < kend_key) ? s[nb][r] : -INFINITY;
         s[nb][r] = sv;
         mx = fmaxf(mx, sv);
       }
@@ -957,18 +1012,18 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
     if (one_by_one) {
       // One chunk at a time: at most one for every wave of the workgroup, or a wide head.
       for (; c0 < stop; c0 += kStride) {
-        RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
-        RLIS_DEC_PAGES(c0 + kStride, pk_a, pv_a);
-        compute(c0, k_a, v_a);
+        RLIS_DEC_CHUNK(RLIS_KEY_AT(c0), pk_a, pv_a, k_a, v_a);
+        RLIS_DEC_PAGES(RLIS_KEY_AT(c0 + kStride), pk_a, pv_a);
+        compute(RLIS_KEY_AT(c0), k_a, v_a);
       }
     } else if constexpr (kPairs) {
       for (; c0 < stop; c0 += 2 * kStride) {
-        RLIS_DEC_CHUNK(c0, pk_a, pv_a, k_a, v_a);
-        RLIS_DEC_CHUNK(c0 + kStride, pk_b, pv_b, k_b, v_b);
-        RLIS_DEC_PAGES(c0 + 2 * kStride, pk_a, pv_a);
-        RLIS_DEC_PAGES(c0 + 3 * kStride, pk_b, pv_b);
-        compute(c0, k_a, v_a);
-        if (c0 + kStride < kend) compute(c0 + kStride, k_b, v_b);
+        RLIS_DEC_CHUNK(RLIS_KEY_AT(c0), pk_a, pv_a, k_a, v_a);
+        RLIS_DEC_CHUNK(RLIS_KEY_AT(c0 + kStride), pk_b, pv_b, k_b, v_b);
+        RLIS_DEC_PAGES(RLIS_KEY_AT(c0 + 2 * kStride), pk_a, pv_a);
+        RLIS_DEC_PAGES(RLIS_KEY_AT(c0 + 3 * kStride), pk_b, pv_b);
+        compute(RLIS_KEY_AT(c0), k_a, v_a);
+        if (c0 + kStride < kend) compute(RLIS_KEY_AT(c0 + kStride), k_b, v_b);
       }
     }
     if (!WALKS || stop >= kend) break;
@@ -982,6 +1037,7 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
   }
 #undef RLIS_DEC_CHUNK
 #undef RLIS_DEC_PAGES
+#undef RLIS_KEY_AT
 
   // ---- the workgroup's last key: merge the waves of every partition, then store ---------
   park(kept);                    // kept = mine - 1
@@ -994,6 +1050,14 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
       // one partition: the sequence's only one, or one to hand over
       merged(0, hh, j, a, big, lsum);
       if (own == 1) {
+        if (sinks) {
+          // e^sink joins the denominator once (the maxima here are base-2 exponents)
+          const float sink2 = sinks[h] * 1.4426950408889634f;
+          const float top = fmaxf(big, sink2);
+          const float e = __builtin_amdgcn_exp2f(big - top);
+          a *= e;
+          lsum = lsum * e + __builtin_amdgcn_exp2f(sink2 - top);
+        }
         out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
       } else {
         const long long idx = ((long long)seq * nh + h) * splits + first;
@@ -1021,6 +1085,14 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
           l_all += lsum * e;
           a_all += a * e;
         }
+      }
+      if (sinks) {
+        // as attn_reduce_kernel adds it: one more partition with e^sink and no values
+        const float sink = sinks[h];
+        const float both = fmaxf(top, sink);
+        const float e = expf(top - both);
+        a_all *= e;
+        l_all = l_all * e + expf(sink - both);
       }
       out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a_all / l_all);
     } else {
@@ -1097,6 +1169,13 @@ __global__ __launch_bounds__(512, RLIS_HEAD_DIM <= 64 ? 4 : 2) void DECODE_KERNE
         a += v * e;
       }
     }
+    if (sinks) {
+      const float sink = sinks[h];
+      const float both = fmaxf(big, sink);
+      const float e = expf(big - both);
+      a *= e;
+      lsum = lsum * e + expf(sink - both);
+    }
     out[(long long)seq * out_stride + h * d + j] = f32_to_bf16(a / lsum);
   }
 }
@@ -1107,7 +1186,8 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
     int max_pages, const int* ctx_lens, int S, int nh, int nkv, int d, int page_shift, int window,
     float scale, int splits, int part_keys, int max_parts, int merge_inside, int groups, int cap,
     const DecodeRope* rope, const DecodeMerge* merge, const float* slopes,
-    const float* head_scales, float softcap, hipStream_t stream) {
+    const float* head_scales, float softcap, const float* sinks, int keep_first,
+    hipStream_t stream) {
   if (S == 0) return 0;
   const bool shaped = slopes || head_scales || softcap > 0.f;
   if (part_keys % (32 * kDecodeWaves) != 0 || part_keys <= 0) return kUnitBadPartition;
@@ -1151,7 +1231,7 @@ RLIS_API int RLIS_CAT(rlis_attn_decode_mfma_d, RLIS_HEAD_DIM)(
       (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, part_ml, part_acc,                   \
       (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, max_pages, ctx_lens, nh, nkv, \
       d, page_shift, scale, window, splits, part_keys, max_parts, merge_inside, groups, cap,   \
-      *rope, *merge, slopes, head_scales, softcap)
+      *rope, *merge, slopes, head_scales, softcap, sinks, keep_first)
   const bool exact = d == D && page_shift == kExactPageShift && window <= 0;
   if (shaped && cap > 1) RLIS_DEC_LAUNCH(true, false, true);
   else if (shaped) RLIS_DEC_LAUNCH(false, false, true);

@@ -977,8 +977,9 @@ def _prefill_mfma_ok(qkv: torch.Tensor, d: int, page_size: int) -> bool:
 # Whether scores with a scale per head or a cap take the matrix-core kernels (False: the
 # vector-unit kernels, for tests that hold the two against each other).
 SHAPED_SCORES_MATRIX = True
-# Whether a sink in the softmax or kept first keys send a batch to the vector-unit kernels.
-PLAIN_EXTRAS = True
+# Whether a sink in the softmax or kept first keys send a batch to the vector-unit kernels
+# (the matrix-core kernels take both; tests hold the two against each other).
+PLAIN_EXTRAS = False
 
 
 def attention_planner(num_heads: int, num_kv_heads: int, head_dim: int,
@@ -1237,7 +1238,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                      nh, nkv, d, page_size, win, float(scale), depth, ap.DECODE_PART_KEYS,
                      ap.DECODE_MAX_PARTS, arrivals_p, arrival_slots, groups, cap, cos_p, sin_p,
                      rot, pos_p, slots_p, nh * d, (nh + nkv) * d, slopes_ptr, scales_ptr, softcap,
-                     stream)
+                     sinks_ptr, kept, stream)
         else:
             lib.call("rlis_attn_decode", qkv.data_ptr(), _dt(qkv), q_stride, out.data_ptr(),
                      nh * d, ml_ptr, acc_ptr, k_pages.data_ptr(), v_pages.data_ptr(),
@@ -1294,7 +1295,7 @@ def paged_attention(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                  _i32(step.start_pos, "start_pos", step.num_seqs),
                  _i32(plan[name], name, 4 * n), n, nh, nkv, d, page_size, win, float(scale), tile,
                  max_runs, row0, ml_ptr, acc_ptr, cos_p, sin_p, rot, slopes_ptr, scales_ptr,
-                 softcap, stream)
+                 softcap, sinks_ptr, kept, stream)
     if not launched and T > row0:
         raise KernelError("attention: the plan holds no tiles for the step's portions")
     if launched and max_runs > 1:
