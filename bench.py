@@ -49,7 +49,13 @@ a cached latent, selective scan, a routed feed-forward; of the experts' weights 
 those that its tokens reach on average, and of a windowed cache the window).
 ``--design lagedra`` times the Lagedra design (three layers of linear attention with a fixed
 decay per head to one of windowed softmax attention behind short convolutions, feed-forwards
-that alternate between a routed mixture and a dense GELU unit)."""
+that alternate between a routed mixture and a dense GELU unit).
+``--design pamolix`` times the Pamolix design (two residual streams mixed by hyper-connections;
+layers alternate between attention over every earlier key with biases, head norms and a sink,
+every second of them on the keys and values of the one before, and attention with a window of
+1,024 that also keeps the first 64 keys, with a gate per head; feed-forwards alternate between a
+dense GELU unit and a mixture of squared-ReLU units).  ``--design lagedra,pamolix`` puts it
+beside its closest kin."""
 import argparse
 import copy
 import json
@@ -277,6 +283,36 @@ def lagedra_like(cfg: dict) -> dict:
             "layers": layers}
 
 
+def pamolix_like(cfg: dict) -> dict:
+    """A Pamolix configuration at the sizes of a Llama preset: the same width, depth, vocabulary,
+    heads and head size; two residual streams; even layers see every earlier key (biased
+    projections, head norms, the queries' factor, a sink), and every second of them reads the
+    keys and values of the one before it; odd layers have a window of 1,024 that keeps the first
+    64 keys, whole-head rotation with positions stretched by 4, capped scores and a gate per
+    head; feed-forwards alternate between a dense GELU unit of one and a half times the preset's
+    width and a mixture of 32 squared-ReLU units (three eighths of the preset's feed-forward
+    width each, four chosen): as many active feed-forward weights per token as the preset has."""
+    W, d, H = cfg["hidden_size"], cfg["head_dim"], cfg["num_attention_heads"]
+    G, ff = cfg["num_key_value_heads"], cfg["intermediate_size"]
+    moe = {"kind": "moe", "expert": {"ff": ff * 3 // 8}, "router": {"experts": 32, "top": 4}}
+    dense = {"kind": "dense", "ff": ff * 3 // 2}
+    first = {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5,
+             "q_temp": {"coef": 0.1, "every": 1024}}
+    second = {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5,
+              "mask": {"size": 1024, "keep_first": 64}, "softcap": 30.0,
+              "rot": {"dims": d, "base": cfg["rope_theta"], "scaling": {"factor": 4.0}}}
+    layers = []
+    for i in range(cfg["num_hidden_layers"]):
+        if i % 2 == 0:
+            mixer = dict(first, kv_from=i - 2) if i % 4 == 2 else dict(first)
+            layers.append({"type": "attention", "mixer": mixer, "mlp": copy.deepcopy(dense)})
+        else:
+            layers.append({"type": "attention_2", "mixer": copy.deepcopy(second),
+                           "mlp": copy.deepcopy(moe)})
+    return {"architecture": "Pamolix", "vocab": cfg["vocab_size"], "width": W,
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "streams": 2, "layers": layers}
+
+
 def step_bytes_of(model, batch: int, mean_context: float) -> float:
     """What a decode step of any model has to move: every tensor its parts hold once (the
     embedding table only where the head shares it), each live request's cached positions, and
@@ -308,7 +344,8 @@ def routed_idle_bytes(model, batch: int) -> float:
         ff = getattr(layer, "feed_forward", None)
         if ff is not None and hasattr(ff, "experts"):
             E = ff.experts
-            per_expert = (ff.w_gate_up.numel() + ff.w_down.numel()) * ff.w_down.element_size() / E
+            up = ff.w_gate_up if hasattr(ff, "w_gate_up") else ff.w_up
+            per_expert = (up.numel() + ff.w_down.numel()) * ff.w_down.element_size() / E
             idle += per_expert * E * (1.0 - 1.0 / E) ** (batch * ff.top)
     return idle
 
@@ -383,7 +420,8 @@ def compare_designs(args) -> int:
             base["num_hidden_layers"] = args.layers
         longest = max(T, args.points_context + new + warm + 16) + 64
         base["max_position_embeddings"] = min(base["max_position_embeddings"], longest)
-        like = {"gipotar": gipotar_like, "bekunex": bekunex_like, "lagedra": lagedra_like}
+        like = {"gipotar": gipotar_like, "bekunex": bekunex_like, "lagedra": lagedra_like,
+                "pamolix": pamolix_like}
         for design, cfg in [("llama", base)] + [(d, like[d](base)) for d in args.design.split(",")]:
             vocab = base["vocab_size"]
             model = random_model(cfg, seed=0, dtype=args.dtype, max_positions=longest)
