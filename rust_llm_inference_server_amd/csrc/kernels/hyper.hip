@@ -90,6 +90,111 @@ __global__ __launch_bounds__(256) void lanes_step_kernel(
   }
 }
 
+// The same step for one to four streams whose rows are a multiple of four wide (what models
+// have): the stream count is a constant of the kernel, so the sums over streams are straight
+// code with every stream's load in flight at once, and a thread moves four columns at a time.
+__device__ __forceinline__ void load4(const float* p, float* o) {
+  const float4 v = *(const float4*)p;
+  o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float* o) {
+  const uint2 v = *(const uint2*)p;
+  o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+  o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float* v) {
+  *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float* v) {
+  uint2 o;
+  o.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+  o.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+  *(uint2*)p = o;
+}
+
+template <int S, typename TY, typename TW, typename TO>
+__global__ __launch_bounds__(256) void lanes_step4_kernel(
+    const float* __restrict__ src, long long src_stride, float* __restrict__ dst,
+    long long dst_stride, const TY* __restrict__ y, int y_parts, long long y_part_stride,
+    int round16, const float* __restrict__ mix, const float* __restrict__ back,
+    const float* __restrict__ read, const TW* __restrict__ norm_w, float eps,
+    TO* __restrict__ out, const int* __restrict__ rows, int H, int store) {
+  extern __shared__ float u_s[];          // H
+  __shared__ float red[4];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const long long t = rows ? rows[r] : r;
+  float m[S][S], b[S], a[S];
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    b[s] = y ? back[s] : 0.f;
+    a[s] = read ? read[s] : 1.f;
+#pragma unroll
+    for (int to = 0; to < S; ++to) m[s][to] = y ? mix[s * S + to] : 0.f;
+  }
+  float ss = 0.f;
+  for (int j = tid * 4; j < H; j += 1024) {
+    float v[S][4];
+#pragma unroll
+    for (int s = 0; s < S; ++s) load4(src + s * src_stride + t * H + j, v[s]);
+    if (y) {
+      float yy[4];
+      load4(y + t * H + j, yy);
+      for (int p = 1; p < y_parts; ++p) {
+        float more[4];
+        load4(y + p * y_part_stride + t * H + j, more);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yy[e] += more[e];
+      }
+      if (round16) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yy[e] = bf16_to_f32(f32_to_bf16(yy[e]));
+      }
+      float nv[S][4];
+#pragma unroll
+      for (int to = 0; to < S; ++to)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float acc = 0.f;
+#pragma unroll
+          for (int s = 0; s < S; ++s) acc += m[s][to] * v[s][e];
+          nv[to][e] = acc + b[to] * yy[e];
+        }
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[s][e] = nv[s][e];
+        if (store) store4(dst + s * dst_stride + t * H + j, nv[s]);
+      }
+    }
+    if (out) {
+      float u[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float acc = 0.f;
+#pragma unroll
+        for (int s = 0; s < S; ++s) acc += a[s] * v[s][e];
+        u[e] = acc;
+        ss += acc * acc;
+      }
+      store4(u_s + j, u);
+    }
+  }
+  if (!out) return;
+  float inv = 1.0f;
+  if (norm_w) inv = 1.0f / sqrtf(block_sum<256>(ss, red) / (float)H + eps);
+  // (a thread reads back the columns it wrote itself: no barrier is needed for them)
+  for (int j = tid * 4; j < H; j += 1024) {
+    float u[4], w[4];
+    load4(u_s + j, u);
+    if (norm_w) {
+      load4(norm_w + j, w);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) u[e] = u[e] * inv * w[e];
+    }
+    store4(out + (long long)r * H + j, u);
+  }
+}
+
 RLIS_API int rlis_lanes_step(const float* src, long long src_stride, float* dst,
                              long long dst_stride, const void* y, int y_dtype, int y_parts,
                              long long y_part_stride, int round16, const float* mix,
@@ -104,10 +209,25 @@ RLIS_API int rlis_lanes_step(const float* src, long long src_stride, float* dst,
   RLIS_REQUIRE(!(rows && store && y), "lanes_step: picked rows leave the streams as they are");
   if (R == 0) return 0;
   const size_t smem = (size_t)H * 4;
-#define LAUNCH(TY, TW, TO)                                                                    \
-  lanes_step_kernel<TY, TW, TO><<<R, 256, smem, stream>>>(                                    \
+  const bool by4 = S <= 4 && H % 4 == 0 && ((uintptr_t)src % 16) == 0 &&
+                   ((uintptr_t)dst % 16) == 0 && src_stride % 4 == 0 && dst_stride % 4 == 0 &&
+                   ((uintptr_t)y % 16) == 0 && y_part_stride % 4 == 0 &&
+                   ((uintptr_t)norm_w % 16) == 0 && ((uintptr_t)out % 16) == 0;
+#define LAUNCH4(SC, TY, TW, TO)                                                               \
+  lanes_step4_kernel<SC, TY, TW, TO><<<R, 256, smem, stream>>>(                               \
       src, src_stride, dst, dst_stride, (const TY*)y, y_parts, y_part_stride, round16, mix,   \
-      back, read, (const TW*)norm_w, eps, (TO*)out, rows, H, S, store)
+      back, read, (const TW*)norm_w, eps, (TO*)out, rows, H, store)
+#define LAUNCH(TY, TW, TO)                                                                    \
+  do {                                                                                        \
+    if (by4 && S == 1) LAUNCH4(1, TY, TW, TO);                                                \
+    else if (by4 && S == 2) LAUNCH4(2, TY, TW, TO);                                           \
+    else if (by4 && S == 3) LAUNCH4(3, TY, TW, TO);                                           \
+    else if (by4 && S == 4) LAUNCH4(4, TY, TW, TO);                                           \
+    else                                                                                      \
+      lanes_step_kernel<TY, TW, TO><<<R, 256, smem, stream>>>(                                \
+          src, src_stride, dst, dst_stride, (const TY*)y, y_parts, y_part_stride, round16,    \
+          mix, back, read, (const TW*)norm_w, eps, (TO*)out, rows, H, S, store);              \
+  } while (0)
 #define BY_OUT(TY, TW)                                     \
   do {                                                     \
     if (out_dtype == RLIS_BF16) LAUNCH(TY, TW, bf16_t);    \
@@ -122,6 +242,7 @@ RLIS_API int rlis_lanes_step(const float* src, long long src_stride, float* dst,
 #undef BY_W
 #undef BY_OUT
 #undef LAUNCH
+#undef LAUNCH4
   RLIS_LAUNCH_CHECK("lanes_step");
   return 0;
 }
@@ -169,6 +290,65 @@ __global__ __launch_bounds__(64) void head_prepare_kernel(
   }
 }
 
+// bfloat16 rows in steps of 8: LPH lanes share a head, eight numbers each (16-byte accesses), so
+// that a wave takes 64 / LPH heads at once; the sum of squares runs over the head's lanes.
+template <int LPH>
+__global__ __launch_bounds__(256) void head_prepare_bf16x8_kernel(
+    bf16_t* __restrict__ qkv, long long stride, int nh, int nkv, int D, int dim,
+    const float* __restrict__ bias, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    float eps, const int* __restrict__ positions, float temp_coef, int temp_every,
+    long long pairs) {
+  const long long pair = ((long long)blockIdx.x * 256 + threadIdx.x) / LPH;
+  const int sub = threadIdx.x % LPH, j0 = sub * 8;
+  const int heads = nh + 2 * nkv;
+  // (lanes past the last pair work on it again and drop the result: the shuffles below want
+  // every lane of the wave)
+  const bool live = pair < pairs && j0 < D;
+  const long long pr = pair < pairs ? pair : pairs - 1;
+  const int t = (int)(pr / heads), h = (int)(pr % heads);
+  const bool is_q = h < nh, is_v = h >= nh + nkv;
+  const float* w = is_q ? q_w : (is_v ? nullptr : k_w);
+  const bool scaled = is_q && temp_every > 0;
+  bf16_t* row = qkv + (long long)t * stride + (long long)h * D + (j0 < D ? j0 : 0);
+  float x[8];
+  {
+    const uint4 v = *(const uint4*)row;
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __uint_as_float(u[i] << 16);
+      x[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int j = j0 + e;
+    if (bias && j < D) x[e] += bias[(long long)h * D + j];
+    if (j < dim && j0 < D) ss += x[e] * x[e];
+  }
+#pragma unroll
+  for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+  const float f = w ? 1.0f / sqrtf(ss / (float)dim + eps) : 1.0f;
+  const float g = scaled ? 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f)
+                         : 1.0f;
+  if (!live || (!bias && !w && !scaled)) return;
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float r[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int j = j0 + 2 * i + e;
+      float v = x[2 * i + e];
+      if (w) v = j < dim ? v * f * w[j] : 0.f;
+      r[e] = v * g;
+    }
+    o[i] = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
+  }
+  *(uint4*)row = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 RLIS_API int rlis_head_prepare(void* qkv, int dtype, long long stride, int T, int nh, int nkv,
                                int D, int dim, const float* bias, const float* q_w,
                                const float* k_w, float eps, const int* positions,
@@ -179,6 +359,27 @@ RLIS_API int rlis_head_prepare(void* qkv, int dtype, long long stride, int T, in
   RLIS_REQUIRE(nh + 2 * nkv <= 65535, "head_prepare: too many heads");
   RLIS_REQUIRE(temp_every <= 0 || positions, "head_prepare: the queries' factor needs positions");
   if (T == 0) return 0;
+  if (dtype == RLIS_BF16 && D % 8 == 0 && stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0) {
+    const long long pairs = (long long)T * (nh + 2 * nkv);
+    int lph = 1;
+    while (lph * 8 < D) lph *= 2;
+    const long long blocks = ceil_div_ll(pairs * lph, 256);
+    RLIS_REQUIRE(blocks < (1ll << 31), "head_prepare: too many rows");
+#define LAUNCH8(LPH)                                                                         \
+  head_prepare_bf16x8_kernel<LPH><<<(unsigned)blocks, 256, 0, stream>>>(                     \
+      (bf16_t*)qkv, stride, nh, nkv, D, dim, bias, q_w, k_w, eps, positions, temp_coef,      \
+      temp_every, pairs)
+    if (lph <= 1) LAUNCH8(1);
+    else if (lph == 2) LAUNCH8(2);
+    else if (lph == 4) LAUNCH8(4);
+    else if (lph == 8) LAUNCH8(8);
+    else if (lph == 16) LAUNCH8(16);
+    else if (lph == 32) LAUNCH8(32);
+    else LAUNCH8(64);
+#undef LAUNCH8
+    RLIS_LAUNCH_CHECK("head_prepare");
+    return 0;
+  }
   dim3 grid(T, nh + 2 * nkv);
   const int dpl = ceil_div(D, 64);
 #define LAUNCH(TX, DPL)                                                                     \
@@ -219,11 +420,42 @@ __global__ void head_gate_kernel(TX* __restrict__ x, long long x_stride,
   }
 }
 
+// bfloat16 heads in steps of 8: eight numbers a thread, all of one head.
+__global__ void head_gate_bf16x8_kernel(bf16_t* __restrict__ x, long long x_stride,
+                                        const bf16_t* __restrict__ gate, long long gate_stride,
+                                        int nh, int D, long long total8) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long step = (long long)gridDim.x * blockDim.x;
+  const int width8 = nh * D / 8;
+  for (; i < total8; i += step) {
+    const long long t = i / width8;
+    const int c = (int)(i % width8) * 8;
+    const float g = 1.0f / (1.0f + expf(-bf16_to_f32(gate[t * gate_stride + c / D])));
+    bf16_t* p = x + t * x_stride + c;
+    const uint4 v = *(const uint4*)p;
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      o[k] = (uint32_t)f32_to_bf16(__uint_as_float(u[k] << 16) * g) |
+             ((uint32_t)f32_to_bf16(__uint_as_float(u[k] & 0xffff0000u) * g) << 16);
+    *(uint4*)p = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 RLIS_API int rlis_head_gate(void* x, int dtype, long long x_stride, const void* gate,
                             long long gate_stride, int T, int nh, int D, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && nh > 0 && D > 0, "head_gate: bad sizes");
   const long long total = (long long)T * nh * D;
   if (total == 0) return 0;
+  if (dtype == RLIS_BF16 && D % 8 == 0 && x_stride % 8 == 0 && ((uintptr_t)x % 16) == 0) {
+    const long long total8 = total / 8;
+    const int blocks8 = (int)(ceil_div_ll(total8, 256) < 16384 ? ceil_div_ll(total8, 256) : 16384);
+    head_gate_bf16x8_kernel<<<blocks8, 256, 0, stream>>>((bf16_t*)x, x_stride, (const bf16_t*)gate,
+                                                        gate_stride, nh, D, total8);
+    RLIS_LAUNCH_CHECK("head_gate");
+    return 0;
+  }
   const int blocks = (int)(ceil_div_ll(total, 256) < 16384 ? ceil_div_ll(total, 256) : 16384);
   if (dtype == RLIS_F32)
     head_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, x_stride, (const float*)gate,
@@ -250,8 +482,49 @@ __global__ void gelu_erf_kernel(TX* __restrict__ out, const TX* __restrict__ x, 
   }
 }
 
+// bfloat16, eight values a thread (16-byte accesses).  erf by the rational form
+// 1 - (a1 t + ... + a5 t^5) exp(-z^2), t = 1 / (1 + p |z|), whose error stays below 2e-7 (a
+// thousandth of a bfloat16's last digit), with the hardware's exponential and reciprocal: the
+// library's erff costs more instructions than this kernel has time for per value.
+__device__ __forceinline__ float gelu_erf_fast(float v) {
+  const float z = fabsf(v) * 0.7071067811865476f;
+  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+  float poly = fmaf(1.061405429f, t, -1.453152027f);
+  poly = fmaf(poly, t, 1.421413741f);
+  poly = fmaf(poly, t, -0.284496736f);
+  poly = fmaf(poly, t, 0.254829592f);
+  const float tail = poly * t * __builtin_amdgcn_exp2f(-z * z * 1.4426950408889634f);
+  const float erf_abs = 1.0f - tail;
+  return 0.5f * v * (1.0f + (v < 0.f ? -erf_abs : erf_abs));
+}
+
+__global__ void gelu_erf_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ x,
+                                       long long n8) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n8; i += stride) {
+    const uint4 v = *(const uint4*)(x + i * 8);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float lo = gelu_erf_fast(__uint_as_float(w[j] << 16));
+      const float hi = gelu_erf_fast(__uint_as_float(w[j] & 0xffff0000u));
+      o[j] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+    }
+    *(uint4*)(out + i * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 RLIS_API int rlis_gelu_erf(void* out, const void* x, int dtype, long long n, hipStream_t stream) {
   if (n <= 0) return 0;
+  if (dtype == RLIS_BF16 && n % 8 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)x % 16) == 0) {
+    const long long n8 = n / 8;
+    const int blocks8 = (int)(ceil_div_ll(n8, 256) < 16384 ? ceil_div_ll(n8, 256) : 16384);
+    gelu_erf_bf16x8_kernel<<<blocks8, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, n8);
+    RLIS_LAUNCH_CHECK("gelu_erf");
+    return 0;
+  }
   const int blocks = (int)(ceil_div_ll(n, 256) < 16384 ? ceil_div_ll(n, 256) : 16384);
   if (dtype == RLIS_F32)
     gelu_erf_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)x, n);
