@@ -27,7 +27,7 @@ def runtime() -> ctypes.CDLL:
         PI, PL = POINTER(c_int), POINTER(c_longlong)
         sig = {
             "rlis_rt_last_error": (c_char_p, []),
-            "rlis_cache_create": (c_void_p, [c_int, c_int, PI, PI, c_int]),
+            "rlis_cache_create": (c_void_p, [c_int, c_int, PI, PI, c_int, PI]),
             "rlis_cache_destroy": (None, [c_void_p]),
             "rlis_cache_reserve": (c_int, [c_void_p, c_longlong, c_int, PI, c_int, PI]),
             "rlis_cache_advance": (c_int, [c_void_p, c_longlong, c_int]),
@@ -87,9 +87,11 @@ class OutOfPages(Exception):
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """A page group: ``window`` None keeps every position, an integer only the latest ones."""
+    """A page group: ``window`` None keeps every position, an integer only the latest ones and,
+    with ``keep_first``, the first so many positions of every sequence beside them."""
     num_pages: int
     window: Optional[int] = None
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)
@@ -108,7 +110,9 @@ class CacheManager:
         n = len(self.groups)
         windows = (c_int * n)(*[int(g.window or 0) for g in self.groups])
         pages = (c_int * n)(*[int(g.num_pages) for g in self.groups])
-        self._h = rt.rlis_cache_create(self.page_size, n, windows, pages, self.num_state_slots)
+        kept = (c_int * n)(*[int(g.keep_first or 0) for g in self.groups])
+        self._h = rt.rlis_cache_create(self.page_size, n, windows, pages, self.num_state_slots,
+                                       kept)
         if not self._h:
             raise ValueError(rt_error())
         self._copies = (c_int * (3 * 4 * max(1, n)))()

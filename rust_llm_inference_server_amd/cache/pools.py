@@ -48,7 +48,9 @@ def pool_pages(cache_groups: Sequence, act_dtype: torch.dtype, page_size: int, b
     for i, g in enumerate(cache_groups):
         w = g.request.window
         if w:
-            held = -(-(w + max_batched_tokens) // page_size) + 1
+            # (kept first positions: their pages beside the window's)
+            held = -(-(w + max_batched_tokens) // page_size) + 1 \
+                + -(-int(getattr(g.request, "keep_first", 0)) // page_size)
             pages[i] = min(even, max(for_one, max_num_seqs * held))
             left -= pages[i] * per_page[i]
         else:

@@ -298,14 +298,16 @@ __global__ __launch_bounds__(256) void head_prepare_bf16x8_kernel(
     const float* __restrict__ bias, const float* __restrict__ q_w, const float* __restrict__ k_w,
     float eps, const int* __restrict__ positions, float temp_coef, int temp_every,
     long long pairs) {
-  const long long pair = ((long long)blockIdx.x * 256 + threadIdx.x) / LPH;
+  // (32-bit arithmetic: the host sees to it that the pairs fit, and a 64-bit division costs more
+  // than everything else here)
+  const unsigned pair = (blockIdx.x * 256u + threadIdx.x) / LPH;
   const int sub = threadIdx.x % LPH, j0 = sub * 8;
-  const int heads = nh + 2 * nkv;
+  const unsigned heads = nh + 2 * nkv;
   // (lanes past the last pair work on it again and drop the result: the shuffles below want
   // every lane of the wave)
   const bool live = pair < pairs && j0 < D;
-  const long long pr = pair < pairs ? pair : pairs - 1;
-  const int t = (int)(pr / heads), h = (int)(pr % heads);
+  const unsigned pr = pair < pairs ? pair : (unsigned)pairs - 1;
+  const int t = (int)(pr / heads), h = (int)(pr - (unsigned)t * heads);
   const bool is_q = h < nh, is_v = h >= nh + nkv;
   const float* w = is_q ? q_w : (is_v ? nullptr : k_w);
   const bool scaled = is_q && temp_every > 0;
@@ -364,7 +366,7 @@ RLIS_API int rlis_head_prepare(void* qkv, int dtype, long long stride, int T, in
     int lph = 1;
     while (lph * 8 < D) lph *= 2;
     const long long blocks = ceil_div_ll(pairs * lph, 256);
-    RLIS_REQUIRE(blocks < (1ll << 31), "head_prepare: too many rows");
+    RLIS_REQUIRE(blocks * 256 < (1ll << 31), "head_prepare: too many rows");
 #define LAUNCH8(LPH)                                                                         \
   head_prepare_bf16x8_kernel<LPH><<<(unsigned)blocks, 256, 0, stream>>>(                     \
       (bf16_t*)qkv, stride, nh, nkv, D, dim, bias, q_w, k_w, eps, positions, temp_coef,      \
@@ -426,12 +428,13 @@ __global__ void head_gate_bf16x8_kernel(bf16_t* __restrict__ x, long long x_stri
                                         int nh, int D, long long total8) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   const long long step = (long long)gridDim.x * blockDim.x;
-  const int width8 = nh * D / 8;
+  const unsigned width8 = nh * D / 8;
   for (; i < total8; i += step) {
-    const long long t = i / width8;
-    const int c = (int)(i % width8) * 8;
-    const float g = 1.0f / (1.0f + expf(-bf16_to_f32(gate[t * gate_stride + c / D])));
-    bf16_t* p = x + t * x_stride + c;
+    // (the host keeps total8 below 2^31: 32-bit division)
+    const unsigned t = (unsigned)i / width8;
+    const int c = (int)((unsigned)i - t * width8) * 8;
+    const float g = 1.0f / (1.0f + expf(-bf16_to_f32(gate[(long long)t * gate_stride + c / D])));
+    bf16_t* p = x + (long long)t * x_stride + c;
     const uint4 v = *(const uint4*)p;
     const uint32_t u[4] = {v.x, v.y, v.z, v.w};
     uint32_t o[4];
@@ -448,7 +451,8 @@ RLIS_API int rlis_head_gate(void* x, int dtype, long long x_stride, const void* 
   RLIS_REQUIRE(T >= 0 && nh > 0 && D > 0, "head_gate: bad sizes");
   const long long total = (long long)T * nh * D;
   if (total == 0) return 0;
-  if (dtype == RLIS_BF16 && D % 8 == 0 && x_stride % 8 == 0 && ((uintptr_t)x % 16) == 0) {
+  if (dtype == RLIS_BF16 && D % 8 == 0 && x_stride % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+      total / 8 < (1ll << 31)) {
     const long long total8 = total / 8;
     const int blocks8 = (int)(ceil_div_ll(total8, 256) < 16384 ? ceil_div_ll(total8, 256) : 16384);
     head_gate_bf16x8_kernel<<<blocks8, 256, 0, stream>>>((bf16_t*)x, x_stride, (const bf16_t*)gate,

@@ -1,6 +1,7 @@
 // C entry points of the host runtime (page manager and scheduler) for the Python binding.
 // Handles are opaque pointers; functions return a negative value and keep a message for
 // rlis_rt_last_error() when an argument is wrong or an internal check fails.
+#include <algorithm>
 #include <cstring>
 #include <exception>
 #include <string>
@@ -36,10 +37,12 @@ static int copy_message(const std::string& msg, char* buf, int cap) {
 
 // ------------------------------------------------------------------------ cache
 RT_API void* rlis_cache_create(int page_size, int num_groups, const int* windows,
-                               const int* num_pages, int num_state_slots) {
+                               const int* num_pages, int num_state_slots,
+                               const int* keep_first) {
   try {
     std::vector<rlis::GroupSpec> groups;
-    for (int g = 0; g < num_groups; ++g) groups.push_back({windows[g], num_pages[g]});
+    for (int g = 0; g < num_groups; ++g)
+      groups.push_back({windows[g], num_pages[g], keep_first ? keep_first[g] : 0});
     return new CacheManager(page_size, groups, num_state_slots);
   } catch (const std::exception& e) {
     g_error = e.what();
@@ -150,8 +153,7 @@ RT_API int rlis_cache_decode_batch(void* h, const long long* seqs, int n, int wi
         return -1;
       }
       int* row = tables[g] + (long long)i * width;
-      for (int p = 0; p < run.gone; ++p) row[p] = 0;
-      for (size_t p = 0; p < run.live.size(); ++p) row[run.gone + p] = run.live[p];
+      for (int p = 0; p < run.count(); ++p) row[p] = std::max(run.at(p), 0);
       const int page = run.at(pos / ps);
       if (page < 0) {
         g_error = "request " + std::to_string(seqs[i]) + ": position " + std::to_string(pos) +

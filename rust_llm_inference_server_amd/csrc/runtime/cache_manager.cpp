@@ -53,7 +53,8 @@ CacheManager::CacheManager(int page_size, std::vector<GroupSpec> groups, int num
   if (page_size_ <= 0) throw std::invalid_argument("page_size must be positive");
   if (groups_.empty()) throw std::invalid_argument("at least one page group is needed");
   for (const GroupSpec& g : groups_) {
-    if (g.num_pages < 0 || g.window < 0) throw std::invalid_argument("bad page group");
+    if (g.num_pages < 0 || g.window < 0 || g.keep_first < 0)
+      throw std::invalid_argument("bad page group");
     pools_.emplace_back(g.num_pages);
   }
   for (int seat = num_seats_ - 1; seat >= 0; --seat) free_seats_.push_back(seat);   // seat 0 on top
@@ -86,7 +87,7 @@ Quote CacheManager::quote(SeqId s, int total_tokens) const {
       // pages that the range [computed, total) lands in and that someone else holds too
       const PageRun& run = l->runs[g];
       const int last = std::min(have, pages_for(total_tokens));
-      for (int i = std::max(l->computed / page_size_, run.gone); i < last; ++i)
+      for (int i = std::max(l->computed / page_size_, run.behind_gap()); i < last; ++i)
         if (pools_[g].refs(run.at(i)) > 1) ++need;
     }
     q.pages[g] = need;
@@ -113,6 +114,8 @@ ReserveResult CacheManager::reserve(SeqId s, int total_tokens, std::vector<PageC
   Lease& l = leases_[s];
   if (l.runs.empty()) {
     l.runs.resize(num_groups());
+    for (int g = 0; g < num_groups(); ++g)
+      l.runs[g].head = groups_[g].window > 0 ? pages_for(groups_[g].keep_first) : 0;
     if (q.seat) {
       l.seat = free_seats_.back();
       free_seats_.pop_back();
@@ -124,8 +127,8 @@ ReserveResult CacheManager::reserve(SeqId s, int total_tokens, std::vector<PageC
     PagePool& pool = pools_[g];
     if (total_tokens > l.computed) {
       const int last = std::min(run.count(), pages_for(total_tokens));
-      for (int i = std::max(l.computed / page_size_, run.gone); i < last; ++i) {
-        int& page = run.live[i - run.gone];
+      for (int i = std::max(l.computed / page_size_, run.behind_gap()); i < last; ++i) {
+        int& page = run.live[run.place(i)];
         if (pool.refs(page) > 1) {
           const int own = pool.take();
           if (copies) copies->push_back(PageCopy{g, page, own});
@@ -151,12 +154,13 @@ void CacheManager::advance(SeqId s, int computed) {
   l.computed = computed;
   for (int g = 0; g < num_groups(); ++g) {
     PageRun& run = l.runs[g];
+    // logical pages [head + gone, keep_from) go: in `live` they stand behind the head pages
     const int keep_from = std::min(first_visible_page(computed, g), run.count());
-    const int passed = keep_from - run.gone;
+    const int passed = keep_from - run.head - run.gone;
     if (passed <= 0) continue;
-    for (int i = 0; i < passed; ++i) pools_[g].drop(run.live[i]);
-    run.live.erase(run.live.begin(), run.live.begin() + passed);
-    run.gone = keep_from;
+    for (int i = 0; i < passed; ++i) pools_[g].drop(run.live[run.head + i]);
+    run.live.erase(run.live.begin() + run.head, run.live.begin() + run.head + passed);
+    run.gone += passed;
   }
 }
 
@@ -173,10 +177,15 @@ std::pair<int, int> CacheManager::fork(SeqId parent, SeqId child) {
   for (int g = 0; g < num_groups(); ++g) {
     const PageRun& src = from.runs[g];
     PageRun& dst = to.runs[g];
-    dst.gone = std::min(src.gone, pages);
-    for (int i = dst.gone; i < pages; ++i) {
-      pools_[g].share(src.at(i));
-      dst.live.push_back(src.at(i));
+    dst.head = src.head;
+    for (int i = 0; i < pages; ++i) {
+      const int page = src.at(i);
+      if (page < 0) {
+        ++dst.gone;
+        continue;
+      }
+      pools_[g].share(page);
+      dst.live.push_back(page);
     }
   }
   if (num_seats_ > 0) {
@@ -215,9 +224,10 @@ std::string CacheManager::audit() const {
         return who(entry.first, g) + ": " + std::to_string(run.count()) + " pages back " +
                std::to_string(l.reserved) + " positions";
       const int visible = std::min(first_visible_page(l.computed, g), run.count());
-      if (run.gone != visible)
-        return who(entry.first, g) + ": pages up to " + std::to_string(run.gone) +
-               " are gone, the window has passed " + std::to_string(visible);
+      if (run.gone != std::max(0, visible - run.head))
+        return who(entry.first, g) + ": " + std::to_string(run.gone) + " pages behind the first " +
+               std::to_string(run.head) + " are gone, the window has passed " +
+               std::to_string(visible);
       for (int p : run.live) {
         if (p < 0 || p >= pool.size())
           return who(entry.first, g) + ": holds page " + std::to_string(p) + ", which does not exist";

@@ -60,17 +60,32 @@ class PagePool {
 };
 
 struct GroupSpec {
-  int window;      // 0: every position is kept; w > 0: only the last w positions
+  int window;          // 0: every position is kept; w > 0: only the last w positions ...
   int num_pages;
+  int keep_first = 0;  // ... and, with a window, the first keep_first positions of the sequence
 };
 
-// The pages of one group that back a request: logical page i is gone (returned, a window has
-// passed it) for i < gone, else live[i - gone].
+// The pages of one group that back a request.  The first `head` logical pages (those that hold
+// positions a window never passes: the sequence's kept first positions) stay for good; of the
+// pages behind them, `gone` have been returned (a window has passed them); `live` holds the
+// pages that are there, in logical order: logical page i is live[i] for i < head (or while
+// nothing is gone), gone for head <= i < head + gone, else live[i - gone].
 struct PageRun {
+  int head = 0;
   int gone = 0;
   std::vector<int> live;
   int count() const { return gone + (int)live.size(); }
-  int at(int i) const { return i < gone ? -1 : live[i - gone]; }
+  // index into live of logical page i, -1 when it is gone
+  int place(int i) const {
+    if (gone == 0 || i < head) return i;
+    return i < head + gone ? -1 : i - gone;
+  }
+  int at(int i) const {
+    const int p = place(i);
+    return p < 0 ? -1 : live[p];
+  }
+  // the first logical page behind the gap (0 when nothing is gone)
+  int behind_gap() const { return gone == 0 ? 0 : head + gone; }
 };
 
 struct Lease {
@@ -98,6 +113,7 @@ class CacheManager {
   int num_free(int g) const { return pools_[g].free_count(); }
   int refcount(int g, int p) const { return pools_[g].refs(p); }
   int window(int g) const { return groups_[g].window; }
+  int keep_first(int g) const { return groups_[g].keep_first; }
   int num_state_slots() const { return num_seats_; }
   int num_free_slots() const { return (int)free_seats_.size(); }
   int pages_for(int tokens) const { return (tokens + page_size_ - 1) / page_size_; }

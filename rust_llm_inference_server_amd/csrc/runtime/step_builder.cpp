@@ -97,7 +97,8 @@ void fill_step(const CacheManager& cache, const std::vector<StepEntryView>& entr
       const PageRun& run = l->runs[g];
       int* slots = buf + lay.offsets[kFixedArrays + 2 * g];
       int* table = buf + lay.offsets[kFixedArrays + 2 * g + 1] + (long long)s * lay.widths[g];
-      for (size_t p = 0; p < run.live.size(); ++p) table[run.gone + p] = std::max(run.live[p], 0);
+      // (pages that are gone read as page 0: kernels load whole tiles and mask what lies in the gap)
+      for (int p = 0; p < run.count(); ++p) table[p] = std::max(run.at(p), 0);
       for (int t = 0; t < e.count; ++t) {
         const int pos = l->computed + t, index = pos / ps;
         const int page = index < run.count() ? run.at(index) : -1;

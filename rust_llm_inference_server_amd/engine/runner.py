@@ -118,7 +118,8 @@ class ModelRunner:
             if len(per_group) != max(1, len(model.cache_groups)):
                 raise ValueError(f"{len(per_group)} pool sizes for "
                                  f"{len(model.cache_groups)} page groups")
-        groups = [GroupSpec(n, g.request.window) for n, g in zip(per_group, model.cache_groups)]
+        groups = [GroupSpec(n, g.request.window, g.request.keep_first)
+                  for n, g in zip(per_group, model.cache_groups)]
         if not groups:
             groups = [GroupSpec(per_group[0], None)]   # the manager always has one group
         self.cache = CacheManager(page_size, groups,

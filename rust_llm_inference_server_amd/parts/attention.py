@@ -51,8 +51,8 @@ class PagedAttention(Mixer):
     * ``sinks``: the name of a tensor with one number per query head: the softmax's denominator
       also holds ``e^sink``, once, unscaled, with no key and no value behind it.
     * ``keep_first`` n (with a ``window``): the first n keys of a sequence stay visible to every
-      later query beside the window's keys, at their own positions.  The cache then keeps every
-      position of such a layer.
+      later query beside the window's keys, at their own positions; the cache keeps their pages
+      while it gives back those that the window has passed.
     * ``gate``: the name of a projection ``(num_heads, hidden_size)`` of the mixer's input: head
       h of the result is multiplied by the sigmoid of output h, in front of the output
       projection.
@@ -230,9 +230,7 @@ class PagedAttention(Mixer):
             plain=self.sinks is not None or bool(self.keep_first and self.window))
 
     def cache_request(self) -> CacheRequest:
-        # (first keys that stay visible: the pages behind the window are not given back)
-        window = None if self.keep_first else self.window
-        return CacheRequest.kv(self.num_kv_heads, self.head_dim, window)
+        return CacheRequest.kv(self.num_kv_heads, self.head_dim, self.window, self.keep_first)
 
     def step_planner(self):
         return self.planner

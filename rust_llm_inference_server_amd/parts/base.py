@@ -94,6 +94,8 @@ class CacheRequest:
 
     arrays: Tuple[PageArray, ...]
     window: Optional[int] = None
+    # with a window: the first so many positions of a sequence are kept beside the latest ones
+    keep_first: int = 0
 
     def __post_init__(self):
         names = [a.name for a in self.arrays]
@@ -101,14 +103,16 @@ class CacheRequest:
             raise ValueError(f"a cache request needs arrays with distinct names, got {names}")
 
     @classmethod
-    def kv(cls, num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheRequest":
+    def kv(cls, num_kv_heads: int, head_dim: int, window: Optional[int] = None,
+           keep_first: int = 0) -> "CacheRequest":
         """Keys ``[kv head][position][d]`` and values ``[kv head][d][position]`` (values
         transposed inside a page, so that both attention kernels read each as it lies)."""
         return cls((PageArray("k", (num_kv_heads, PAGE, head_dim)),
-                    PageArray("v", (num_kv_heads, head_dim, PAGE))), window)
+                    PageArray("v", (num_kv_heads, head_dim, PAGE))), window,
+                   int(keep_first) if window else 0)
 
     def group_key(self) -> Tuple[Any, ...]:
-        return (self.arrays, self.window)
+        return (self.arrays, self.window, self.keep_first)
 
     def elements_per_token(self) -> int:
         return sum(a.elements_per_token() for a in self.arrays)

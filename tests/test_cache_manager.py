@@ -110,6 +110,37 @@ def test_window_group_gives_pages_back_as_the_window_passes():
     m.check_invariants()
 
 
+def test_window_group_keeps_the_pages_of_the_first_positions():
+    """A window of 6 that also keeps the sequence's first 5 positions: pages 0 and 1 (positions
+    0..7) stay for good, the pages between them and the window go back one by one, a fork
+    shares what is there, and a request shorter than the kept positions loses nothing."""
+    m = CacheManager(4, [GroupSpec(16), GroupSpec(16, window=6, keep_first=5)])
+    m.reserve(1, 30)
+    assert m.num_free_pages(1) == 8
+    m.advance(1, 9)       # position 9 sees 4..9 and 0..4: nothing is dead yet
+    assert m.table(1, 1) == list(range(8)) and m.num_free_pages(1) == 8
+    m.advance(1, 19)      # position 19 sees 14..19 and 0..4: page 2 (8..11) is dead
+    assert m.table(1, 1) == [0, 1, -1, 3, 4, 5, 6, 7] and m.num_free_pages(1) == 9
+    m.check_invariants()
+    m.advance(1, 27)      # position 27 sees 22..27: pages 2, 3, 4 are dead
+    assert m.table(1, 1) == [0, 1, -1, -1, -1, 5, 6, 7] and m.num_free_pages(1) == 11
+    assert m.table(1, 0) == list(range(8))
+    m.check_invariants()
+    m.fork(1, 2)          # shares the computed positions' pages: 0, 1, 5 and 6
+    assert m.table(2, 1) == [0, 1, -1, -1, -1, 5, 6]
+    m.check_invariants()
+    m.reserve(2, 28)      # the child's last page is shared and gets written: a copy first
+    assert m.table(2, 1)[:6] == [0, 1, -1, -1, -1, 5] and m.table(2, 1)[6] not in (6, -1)
+    m.check_invariants()
+    m.reserve(3, 7)       # freed pages are used again
+    m.advance(3, 7)
+    assert -1 not in m.table(3, 1)
+    for seq in (1, 2, 3):
+        m.free(seq)
+    assert m.num_free_pages(0) == 16 and m.num_free_pages(1) == 16
+    m.check_invariants()
+
+
 def test_window_longer_than_the_sequence_keeps_everything():
     m = CacheManager(8, [GroupSpec(4, window=100)])
     m.reserve(1, 30)

@@ -112,7 +112,8 @@ def test_the_runtimes_step_layout_is_the_python_twins():
                              "few": np.asarray(lengths.start, dtype=np.int32)}, {"n": n})
 
     rng = np.random.default_rng(7)
-    cache = CacheManager(8, [GroupSpec(400, None), GroupSpec(400, 24)], num_state_slots=16)
+    cache = CacheManager(8, [GroupSpec(400, None), GroupSpec(400, 24), GroupSpec(400, 20, 11)],
+                         num_state_slots=16)
     cpu = torch.device("cpu")
     planners = [AttentionPlanner(4, 2, 16), Wordy()]
     lengths = {}
