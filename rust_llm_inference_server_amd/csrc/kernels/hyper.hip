@@ -292,58 +292,70 @@ __global__ __launch_bounds__(64) void head_prepare_kernel(
 
 // bfloat16 rows in steps of 8: LPH lanes share a head, eight numbers each (16-byte accesses), so
 // that a wave takes 64 / LPH heads at once; the sum of squares runs over the head's lanes.
-template <int LPH>
+// Whether there is a bias and a norm is known to the compiler, so that no load sits under a
+// condition and all of a lane's loads are on their way before the first is used.
+__device__ __forceinline__ void load8f_at(const float* p, float* o) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+
+template <int LPH, bool BIAS, bool NORM>
 __global__ __launch_bounds__(256) void head_prepare_bf16x8_kernel(
     bf16_t* __restrict__ qkv, long long stride, int nh, int nkv, int D, int dim,
     const float* __restrict__ bias, const float* __restrict__ q_w, const float* __restrict__ k_w,
     float eps, const int* __restrict__ positions, float temp_coef, int temp_every,
     long long pairs) {
-  // (32-bit arithmetic: the host sees to it that the pairs fit, and a 64-bit division costs more
-  // than everything else here)
+  // (32-bit arithmetic: the host sees to it that the pairs fit)
   const unsigned pair = (blockIdx.x * 256u + threadIdx.x) / LPH;
-  const int sub = threadIdx.x % LPH, j0 = sub * 8;
+  const int sub = threadIdx.x % LPH;
   const unsigned heads = nh + 2 * nkv;
-  // (lanes past the last pair work on it again and drop the result: the shuffles below want
-  // every lane of the wave)
-  const bool live = pair < pairs && j0 < D;
+  // (lanes past the last pair, and lanes past the head's width, work on a place that is there
+  // and drop the result: the shuffles below want every lane of the wave)
+  const bool live = pair < pairs && sub * 8 < D;
+  const int j0 = sub * 8 < D ? sub * 8 : 0;
   const unsigned pr = pair < pairs ? pair : (unsigned)pairs - 1;
   const int t = (int)(pr / heads), h = (int)(pr - (unsigned)t * heads);
   const bool is_q = h < nh, is_v = h >= nh + nkv;
-  const float* w = is_q ? q_w : (is_v ? nullptr : k_w);
+  const bool normed = NORM && !is_v && (is_q || k_w != nullptr);
   const bool scaled = is_q && temp_every > 0;
-  bf16_t* row = qkv + (long long)t * stride + (long long)h * D + (j0 < D ? j0 : 0);
+  bf16_t* row = qkv + (long long)t * stride + (long long)h * D + j0;
+  const uint4 raw = *(const uint4*)row;
+  float bv[8], wv[8];
+  if constexpr (BIAS) load8f_at(bias + (long long)h * D + j0, bv);
+  if constexpr (NORM) load8f_at(((is_q || !k_w) ? q_w : k_w) + min(j0, dim - 8), wv);
+  const int pos = temp_every > 0 ? positions[t] : 0;
   float x[8];
-  {
-    const uint4 v = *(const uint4*)row;
-    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+  const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x[2 * i] = __uint_as_float(u[i] << 16);
-      x[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
-    }
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = __uint_as_float(u[i] << 16);
+    x[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
   }
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const int j = j0 + e;
-    if (bias && j < D) x[e] += bias[(long long)h * D + j];
-    if (j < dim && j0 < D) ss += x[e] * x[e];
+    if constexpr (BIAS) x[e] += bv[e];
+    if (j0 + e < dim && live) ss += x[e] * x[e];
   }
+  float f = 1.0f;
+  if constexpr (NORM) {
 #pragma unroll
-  for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
-  const float f = w ? 1.0f / sqrtf(ss / (float)dim + eps) : 1.0f;
-  const float g = scaled ? 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f)
-                         : 1.0f;
-  if (!live || (!bias && !w && !scaled)) return;
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+    f = 1.0f / sqrtf(ss / (float)dim + eps);
+  }
+  const float g = scaled ? 1.0f + temp_coef * logf((float)((pos + 1) / temp_every) + 1.0f) : 1.0f;
+  if (!live || (!BIAS && !normed && !scaled)) return;
   uint32_t o[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     float r[2];
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-      const int j = j0 + 2 * i + e;
       float v = x[2 * i + e];
-      if (w) v = j < dim ? v * f * w[j] : 0.f;
+      if constexpr (NORM) {
+        if (normed) v = j0 + 2 * i + e < dim ? v * f * wv[2 * i + e] : 0.f;
+      }
       r[e] = v * g;
     }
     o[i] = (uint32_t)f32_to_bf16(r[0]) | ((uint32_t)f32_to_bf16(r[1]) << 16);
@@ -361,23 +373,33 @@ RLIS_API int rlis_head_prepare(void* qkv, int dtype, long long stride, int T, in
   RLIS_REQUIRE(nh + 2 * nkv <= 65535, "head_prepare: too many heads");
   RLIS_REQUIRE(temp_every <= 0 || positions, "head_prepare: the queries' factor needs positions");
   if (T == 0) return 0;
-  if (dtype == RLIS_BF16 && D % 8 == 0 && stride % 8 == 0 && ((uintptr_t)qkv % 16) == 0) {
+  if (dtype == RLIS_BF16 && D % 8 == 0 && dim % 8 == 0 && stride % 8 == 0 &&
+      ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)bias % 16) == 0 && ((uintptr_t)q_w % 16) == 0 &&
+      ((uintptr_t)k_w % 16) == 0 && (q_w || !k_w)) {
     const long long pairs = (long long)T * (nh + 2 * nkv);
     int lph = 1;
     while (lph * 8 < D) lph *= 2;
     const long long blocks = ceil_div_ll(pairs * lph, 256);
     RLIS_REQUIRE(blocks * 256 < (1ll << 31), "head_prepare: too many rows");
-#define LAUNCH8(LPH)                                                                         \
-  head_prepare_bf16x8_kernel<LPH><<<(unsigned)blocks, 256, 0, stream>>>(                     \
+#define LAUNCH8(LPH, BIAS, NORM)                                                             \
+  head_prepare_bf16x8_kernel<LPH, BIAS, NORM><<<(unsigned)blocks, 256, 0, stream>>>(         \
       (bf16_t*)qkv, stride, nh, nkv, D, dim, bias, q_w, k_w, eps, positions, temp_coef,      \
       temp_every, pairs)
-    if (lph <= 1) LAUNCH8(1);
-    else if (lph == 2) LAUNCH8(2);
-    else if (lph == 4) LAUNCH8(4);
-    else if (lph == 8) LAUNCH8(8);
-    else if (lph == 16) LAUNCH8(16);
-    else if (lph == 32) LAUNCH8(32);
-    else LAUNCH8(64);
+#define BY_FORM(LPH)                                          \
+  do {                                                        \
+    if (bias && q_w) LAUNCH8(LPH, true, true);                \
+    else if (bias) LAUNCH8(LPH, true, false);                 \
+    else if (q_w) LAUNCH8(LPH, false, true);                  \
+    else LAUNCH8(LPH, false, false);                          \
+  } while (0)
+    if (lph <= 1) BY_FORM(1);
+    else if (lph == 2) BY_FORM(2);
+    else if (lph == 4) BY_FORM(4);
+    else if (lph == 8) BY_FORM(8);
+    else if (lph == 16) BY_FORM(16);
+    else if (lph == 32) BY_FORM(32);
+    else BY_FORM(64);
+#undef BY_FORM
 #undef LAUNCH8
     RLIS_LAUNCH_CHECK("head_prepare");
     return 0;
