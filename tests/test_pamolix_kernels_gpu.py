@@ -88,7 +88,7 @@ def test_attention_with_a_sink_and_kept_first_keys(dtype, nh, nkv, d, ps, monkey
 
 @pytest.mark.parametrize("S", [1, 2, 3, 7])
 @pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T, H", [(1, 40), (9, 256), (70, 100), (5, 4100)])
+@pytest.mark.parametrize("T, H", [(1, 40), (9, 256), (70, 100), (5, 4100), (3, 30), (11, 125)])
 def test_the_residual_streams_step(S, y_dtype, T, H):
     """Update, read-out and norm in one pass and each alone; streams that still share one
     tensor; a result that comes as partial sums; picked rows, which leave the streams alone."""
