@@ -38,6 +38,7 @@ class PamolixMixer:
     # "attention"
     temp_coef: float = 0.0              # queries times 1 + coef ln(floor((p + 1) / every) + 1)
     temp_every: int = 0                 # 0: no such factor
+    # either kind
     kv_from: Optional[int] = None       # layer whose keys and values this one reads
     # "attention_2"
     window: Optional[int] = None        # positions a query sees, itself included
@@ -62,8 +63,6 @@ class PamolixMixer:
                 kw["temp_coef"] = _need(temp, "coef", float, where + " q_temp")
                 kw["temp_every"] = _positive(_need(temp, "every", int, where + " q_temp"),
                                              "every", where + " q_temp")
-            if d.get("kv_from") is not None:
-                kw["kv_from"] = _typed(d["kv_from"], "kv_from", int, where)
         else:
             if d.get("mask") is not None:
                 mask = _obj(d, "mask", where)
@@ -85,6 +84,8 @@ class PamolixMixer:
                 if rot.get("scaling") is not None:
                     kw["rot_factor"] = _need(_obj(rot, "scaling", where + " rot"), "factor",
                                              float, where + " rot scaling")
+        if d.get("kv_from") is not None:
+            kw["kv_from"] = _typed(d["kv_from"], "kv_from", int, where)
         out = cls(**kw)
         if out.heads % out.kv_heads:
             raise ConfigError(f"{where}: 'heads' {out.heads} is not a multiple of 'kv_heads' "
@@ -106,6 +107,8 @@ class PamolixMixer:
             if self.kv_from is not None:
                 d["kv_from"] = self.kv_from
             return d
+        if self.kv_from is not None:
+            d["kv_from"] = self.kv_from
         if self.window is not None:
             d["mask"] = {"keep_first": self.keep_first, "size": self.window}
         if self.softcap:

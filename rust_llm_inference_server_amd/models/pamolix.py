@@ -21,10 +21,25 @@ from ..registry import Architecture, register_architecture
 from .spec import LayerSpec, ModelSpec, RunEntry
 
 
-def _mixer(cfg: PamolixConfig, m: PamolixMixer) -> PartSpec:
+def _kept_by_cache(cfg: PamolixConfig, index: int) -> Optional[dict]:
+    """What the pages of layer ``index`` (or of the layer whose pages it reads) must keep: the
+    widest of the masks of all layers that read them; None when the layer's own mask says it."""
+    owner = cfg.layers[index].mixer.kv_from
+    owner = index if owner is None else owner
+    readers = [l.mixer for i, l in enumerate(cfg.layers) if i == owner or l.mixer.kv_from == owner]
+    if len(readers) == 1:
+        return None
+    if any(m.window is None for m in readers):
+        return {"window": None, "keep_first": 0}
+    return {"window": max(m.window for m in readers),
+            "keep_first": max(m.keep_first for m in readers)}
+
+
+def _mixer(cfg: PamolixConfig, m: PamolixMixer, index: int) -> PartSpec:
     params = {"hidden_size": cfg.width, "num_heads": m.heads, "num_kv_heads": m.kv_heads,
               "head_dim": m.dim, "value_dim": m.vdim, "scale": m.scale,
-              "names": {"q": "q", "k": "k", "v": "v", "o": "o"}}
+              "names": {"q": "q", "k": "k", "v": "v", "o": "o"},
+              "cache_like": _kept_by_cache(cfg, index)}
     if m.kind == "attention":
         params.update({
             "window": None, "position": PartSpec("none"), "bias": ".b",
@@ -39,7 +54,8 @@ def _mixer(cfg: PamolixConfig, m: PamolixMixer) -> PartSpec:
         position = PartSpec("rope", {"rot_dim": m.rot_dims, "theta": m.rot_base,
                                      "scaling": scaling, "precise": True})
     params.update({"window": m.window, "keep_first": m.keep_first if m.window else 0,
-                   "position": position, "softcap": m.softcap or None, "gate": "g"})
+                   "position": position, "softcap": m.softcap or None, "gate": "g",
+                   "shared_kv": m.kv_from is not None})
     return PartSpec("attention", params)
 
 
@@ -62,7 +78,7 @@ def pamolix_spec(cfg: PamolixConfig) -> ModelSpec:
     layers: List[LayerSpec] = []
     runs: List[RunEntry] = []
     for i, layer in enumerate(cfg.layers):
-        params = {"mixer": _mixer(cfg, layer.mixer), "feed_forward": _feed_forward(cfg, layer),
+        params = {"mixer": _mixer(cfg, layer.mixer, i), "feed_forward": _feed_forward(cfg, layer),
                   "mixer_norm": norm, "ffn_norm": norm,
                   "names": {"mixer_norm": "norm1", "mixer": "mix", "ffn_norm": "norm2",
                             "feed_forward": "mlp"}}

@@ -56,6 +56,9 @@ class PagedAttention(Mixer):
     * ``gate``: the name of a projection ``(num_heads, hidden_size)`` of the mixer's input: head
       h of the result is multiplied by the sigmoid of output h, in front of the output
       projection.
+    * ``cache_like``: ``{"window": w or None, "keep_first": n}``: what the cache keeps for this
+      layer's pages when that is more than the layer's own mask sees (a layer whose pages another
+      layer with a wider mask reads, and that reader itself: both name the wider of the two).
     * ``shared_kv``: the layer has no key and value projections (nor what belongs to them:
       biases, the keys' norm); its run reads the cache that another run wrote.
 
@@ -187,6 +190,9 @@ class PagedAttention(Mixer):
         if params.get("sinks"):
             self.sinks = ctx.take(join(prefix, params["sinks"])).to(torch.float32).contiguous()
         self.keep_first = int(params.get("keep_first") or 0)
+        like = params.get("cache_like")
+        self.cache_like = None if like is None else (like.get("window"),
+                                                     int(like.get("keep_first") or 0))
         self.w_o = self._pad_heads(ctx.take(names["o"]), self.num_heads, v_dim, self.head_dim,
                                    rows=False).contiguous()
         self.act_dtype = ctx.act_dtype
@@ -230,6 +236,8 @@ class PagedAttention(Mixer):
             plain=self.sinks is not None or bool(self.keep_first and self.window))
 
     def cache_request(self) -> CacheRequest:
+        if self.cache_like is not None:
+            return CacheRequest.kv(self.num_kv_heads, self.head_dim, *self.cache_like)
         return CacheRequest.kv(self.num_kv_heads, self.head_dim, self.window, self.keep_first)
 
     def step_planner(self):

@@ -6,7 +6,7 @@ in config.json chooses the model everywhere: loader, engine, replay.
 The registry names no architecture itself.  Each architecture registers from its own module
 (``models/llama.py`` does for ``LlamaForCausalLM``); the modules that ship with the package are
 imported, once, at the first lookup."""
-# (models/gipotar.py and models/bekunex.py register ``Gipotar`` and ``Bekunex`` the same way.)
+# (models/gipotar.py, bekunex.py, lagedra.py and pamolix.py register their designs the same way.)
 from __future__ import annotations
 
 import json

@@ -118,18 +118,29 @@ def attention(h: torch.Tensor, m: Dict[str, Any], w: Dict[str, torch.Tensor], pr
     return out.reshape(n, -1) @ w[pre + "o"].T
 
 
-def attention_2(h: torch.Tensor, m: Dict[str, Any], w: Dict[str, torch.Tensor], pre: str
-                ) -> torch.Tensor:
-    """The mixer 'attention_2': rotated queries and keys, capped scores, a window that also
-    keeps the sequence's first keys, a gate per head on the output."""
-    n, H, G = h.shape[0], m["heads"], m["kv_heads"]
-    q, k, v = (_heads(h @ w[pre + name].T, heads) for name, heads in
-               (("q", H), ("k", G), ("v", G)))
+def _rotated(x: torch.Tensor, m: Dict[str, Any]) -> torch.Tensor:
     rot = m.get("rot")
-    if rot:
-        factor = (rot.get("scaling") or {}).get("factor", 1.0)
-        q = rotate_half_pairs(q, rot["dims"], rot["base"], factor)
-        k = rotate_half_pairs(k, rot["dims"], rot["base"], factor)
+    if not rot:
+        return x
+    factor = (rot.get("scaling") or {}).get("factor", 1.0)
+    return rotate_half_pairs(x, rot["dims"], rot["base"], factor)
+
+
+def attention_2_keys_values(h: torch.Tensor, m: Dict[str, Any], w: Dict[str, torch.Tensor],
+                            pre: str):
+    """Keys (rotated) and values of the second kind of attention, as its cache holds them."""
+    G = m["kv_heads"]
+    return _rotated(_heads(h @ w[pre + "k"].T, G), m), _heads(h @ w[pre + "v"].T, G)
+
+
+def attention_2(h: torch.Tensor, m: Dict[str, Any], w: Dict[str, torch.Tensor], pre: str,
+                kv=None) -> torch.Tensor:
+    """The mixer 'attention_2': rotated queries and keys, capped scores, a window that also
+    keeps the sequence's first keys, a gate per head on the output; ``kv``: another layer's
+    keys and values in place of its own."""
+    n, H = h.shape[0], m["heads"]
+    q = _rotated(_heads(h @ w[pre + "q"].T, H), m)
+    k, v = kv if kv is not None else attention_2_keys_values(h, m, w, pre)
     mask = m.get("mask") or {}
     ok = visible(n, mask.get("size"), mask.get("keep_first", 0))
     out = _attend(q, k, v, m["scale"], ok, None, m.get("softcap"))
@@ -174,12 +185,16 @@ def forward(config: Dict[str, Any], weights: Dict[str, torch.Tensor], tokens: Li
         m = layer["mixer"]
 
         def mixer(h):
+            if m.get("kv_from") is not None:
+                kv = kept[m["kv_from"]]
+            elif layer["type"] == "attention":
+                kv = attention_keys_values(h, m, w, pre + "mix.", eps)
+            else:
+                kv = attention_2_keys_values(h, m, w, pre + "mix.")
+            kept[i] = kv
             if layer["type"] == "attention":
-                kv = kept[m["kv_from"]] if m.get("kv_from") is not None else \
-                    attention_keys_values(h, m, w, pre + "mix.", eps)
-                kept[i] = kv
                 return attention(h, m, w, pre + "mix.", eps, kv)
-            return attention_2(h, m, w, pre + "mix.")
+            return attention_2(h, m, w, pre + "mix.", kv)
 
         def feed(h):
             if layer["mlp"]["kind"] == "dense":
