@@ -6,7 +6,10 @@
 //    count as minus infinity); the `top` largest choice scores win (the lower index on a tie);
 //    an expert's weight is its s times `scale`, not renormalised.  One wave per token.
 //    Switches: s = softmax(z) over all experts; a group's score the largest choice score in it;
-//    the chosen experts' weights divided by their sum.  A unit's bounded form: see gated_unit.
+//    the chosen experts' weights divided by their sum; a bias per expert added to the logits in
+//    front of everything (softmax scores over all experts, divided by the chosen ones' sum, are
+//    the softmax over the chosen logits alone).  A unit's bounded form: see gated_unit; units
+//    without a gate (one projection, the square of its ReLU, the down projection): plain_unit.
 //  * moe_sort: the step's (token, choice) pairs ordered by expert, every expert's run padded to
 //    whole tiles of rows, so that a tile has one expert.  Decided on the device: nothing waits
 //    for the host.  Which row of its expert's run a pair gets does not move its result: rows of a
