@@ -21,7 +21,8 @@ from gipotar_models import (as_stored, prompts, row_error, write_folder,  # noqa
 def judge(errors: List[float], dtype: str) -> None:
     """float32: no row beyond two and a half times the tolerance and at most one in fifty beyond
     it.  bfloat16: at most one row in six beyond the tolerance, whatever its size, and the
-    median within a third of it.  Where two experts' logits lie closer than bfloat16 resolves
+    median within half of it (weights made so that one score stands far out carry bfloat16's
+    rounding of that score into every row).  Where two experts' logits lie closer than bfloat16 resolves
     the router's input, the engine may take the other one; that row is then far from the plain
     logits, and so, less far, are the later rows that attend to it (these models route in up to
     three layers, with as few as one expert chosen out of four, and their streams' coefficients
@@ -35,7 +36,7 @@ def judge(errors: List[float], dtype: str) -> None:
     else:
         assert over <= max(1, len(errors) // 6), f"{over} of {len(errors)} rows beyond {tol}"
         median = sorted(errors)[len(errors) // 2]
-        assert median < tol / 3 or len(errors) < 20, f"median of the row errors {median:.3g}"
+        assert median < tol / 2 or len(errors) < 20, f"median of the row errors {median:.3g}"
 
 
 def _moe(ff, experts, top):
