@@ -359,6 +359,8 @@ def test_keys_just_inside_and_outside_every_window(backend, dtype, layer, back,
     positions behind the query: the last one inside or the first one outside (and beyond the
     kept first keys).  A window that is one token off, in a prompt's portion or decoded alone,
     moves the row far."""
+    if backend.type == "cpu" and (layer, back) not in ((1, 19), (3, 16), (5, 33)):
+        pytest.skip("the double takes its time: one edge of every window here, all on the GPU")
     cfg = copy.deepcopy(pm.CONFIG_A)
     size = cfg["layers"][layer]["mixer"]["mask"]["size"]
     w = _attention_stands_out(cfg, _marked(cfg, seed=31 + layer), layer)
@@ -389,6 +391,8 @@ def test_the_last_kept_first_key_and_the_one_behind_it(backend, dtype, layer, at
     the last kept one or the first that is not, far in front of every window that the queries
     (in the prompt's part and decoded) have.  A count of kept keys that is one off moves the
     rows far."""
+    if backend.type == "cpu" and (layer, at) not in ((1, 5), (3, 15)):
+        pytest.skip("the double takes its time: one side of either edge here, all on the GPU")
     cfg = copy.deepcopy(pm.CONFIG_A)
     keep = cfg["layers"][layer]["mixer"]["mask"]["keep_first"]
     w = _attention_stands_out(cfg, _marked(cfg, seed=51 + layer), layer)
@@ -418,6 +422,8 @@ def test_a_far_key_that_stands_out(backend, dtype, layer, far, tmp_path_factory)
     takes most of the weight of queries 100 and more positions on, in a prompt's portion and
     decoded alone.  Were its row lost or read from a wrong page, the layer would return another
     token's value."""
+    if backend.type == "cpu" and (layer, far) not in ((0, 16), (2, 15)):
+        pytest.skip("the double takes its time: a page's two sides here, all on the GPU")
     cfg = copy.deepcopy(pm.CONFIG_A)
     w = _attention_stands_out(cfg, _marked(cfg, seed=41), layer)
     folder, _, stored = model_case("a", dtype, tmp_path_factory, weights=w, tag=f"far{layer}",
