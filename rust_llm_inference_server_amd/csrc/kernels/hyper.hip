@@ -139,11 +139,19 @@ __global__ __launch_bounds__(256) void lanes_step4_kernel(
     if (y) {
       float yy[4];
       load4(y + t * H + j, yy);
-      for (int p = 1; p < y_parts; ++p) {
-        float more[4];
-        load4(y + p * y_part_stride + t * H + j, more);
+      // further parts four at a time, asked for together (one past the last reads the last
+      // again and is dropped), added in their order
+      for (int p = 1; p < y_parts; p += 4) {
+        float more[4][4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) yy[e] += more[e];
+        for (int q = 0; q < 4; ++q)
+          load4(y + (long long)min(p + q, y_parts - 1) * y_part_stride + t * H + j, more[q]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (p + q < y_parts) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) yy[e] += more[q][e];
+          }
       }
       if (round16) {
 #pragma unroll
